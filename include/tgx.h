@@ -27,7 +27,7 @@ extern "C" {
 
 /* 3 (round 5): per-row sequence lifecycle (tgx_reset_row / tgx_forward_row / tgx_sample_row / tgx_past_length_row); tgx_get_option added and
  * tgx_engine_read_stats + the options engine.*, pf.*, attn.fold_*, lmhead.fuse_finalize removed since 2. */
-#define TGX_ABI_VERSION 3
+#define TGX_ABI_VERSION 4   /* 4: layered models (tgx_create_stack, tgx_step_ragged) */
 
 #if defined(__GNUC__)
 #define TGX_API __attribute__((visibility("default")))
@@ -55,7 +55,8 @@ typedef enum tgx_family {
   TGX_FAMILY_LLAMA = 2,
   TGX_FAMILY_QWEN2 = 3,
   TGX_FAMILY_QWEN3 = 4,
-  TGX_FAMILY_MISTRAL = 5
+  TGX_FAMILY_MISTRAL = 5,
+  TGX_FAMILY_ZAKUSUN = 6   /* a layered model (tgx_stack_desc below), no counterpart in the reference */
 } tgx_family;
 
 /* tinytorch::DType values the CLI accepts (examples/inference/main.cpp:82-88) */
@@ -90,6 +91,53 @@ typedef struct tgx_model_desc {
                           /*    src/layer/Attention.h:128-167; Qwen3, ModelQwen3.h:23-40)        */
 } tgx_model_desc;
 
+/* ---- layered models (ABI 4) ----------------------------------------------------------------
+ * A model whose config.json lists its layers one by one, each with its own mixer and feed-forward sizes, does not fit the flat
+ * tgx_model_desc: it is described by one tgx_stack_desc and an array of tgx_layer_desc, created by tgx_create_stack, and served by the
+ * same calls as the other families (tgx_upload by checkpoint name, tgx_finalize, tgx_forward / tgx_forward_row, tgx_sample*, tgx_decode,
+ * tgx_step_async, tgx_reset_row / tgx_reset_cache, tgx_read_logits) plus tgx_step_ragged.  Its rows are sequence slots: a slot holds the
+ * short-convolution inputs of every sublayer and a table of pages of the shared latent cache pool.
+ * Mechanisms (each a parameterised building block of csrc/kernels/stack*.h):
+ *   grouped RMS norm          the vector in norm_groups equal parts, each divided by its own sqrt(mean(part^2) + norm_eps), times a weight
+ *   input convolution         every sublayer reads h + conv(h), conv a causal depth-wise filter of canon_taps taps over the normed inputs
+ *   latent attention          queries per head against a shared low-rank latent (the only cached quantity), softmax with a learned per-head
+ *                             sink in the denominator, sigmoid output gate
+ *   mixture of experts        top-k of a 32-bit router (+ bias), weights = softmax over the chosen logits, clamped gated experts
+ *   depth average             the stream handed to layer i + 1 is a learned weighting of the embedding output and all layer results so far
+ *   sinusoidal positions      added to the embedding rows (interleaved sin / cos, base 10000) */
+typedef enum tgx_mixer { TGX_MIXER_LATENT_ATTENTION = 1 } tgx_mixer;
+typedef enum tgx_mlp { TGX_MLP_NONE = 0, TGX_MLP_MOE = 1 } tgx_mlp;
+
+typedef struct tgx_layer_desc {
+  int32_t mixer;     /* tgx_mixer                                                                 */
+  int32_t heads;     /* query heads                                                               */
+  int32_t dim;       /* query / key dimensions per head                                           */
+  int32_t vdim;      /* value dimensions per head                                                 */
+  int32_t kv_rank;   /* width of the cached latent                                                */
+  float scale;       /* score scale                                                               */
+  int32_t mlp;       /* tgx_mlp                                                                   */
+  int32_t experts;   /* experts of the layer                                                      */
+  int32_t top;       /* experts per token                                                         */
+  int32_t ff;        /* expert width                                                              */
+  float limit;       /* clamp of the expert's gate (from above) and up (both sides) projections   */
+} tgx_layer_desc;
+
+typedef struct tgx_stack_desc {
+  int32_t family;         /* tgx_family (TGX_FAMILY_ZAKUSUN)                                       */
+  int32_t width;          /* residual width                                                        */
+  int32_t layers;         /* entries of the tgx_layer_desc array                                   */
+  int32_t vocab;
+  int32_t compute_dtype;  /* tgx_dtype of the stored matrices and of the latent cache              */
+  int32_t max_seqs;       /* sequence slots (rows)                                                 */
+  int32_t max_ctx;        /* longest sequence a slot may hold                                      */
+  int32_t budget_tokens;  /* tokens of the latent cache pool all slots share (<= 0: max_seqs * max_ctx) */
+  int32_t page_tokens;    /* tokens per page of that pool, a power of two (<= 0: 64)               */
+  int32_t norm_groups;
+  float norm_eps;
+  int32_t canon_taps;     /* taps of the input convolution (>= 1)                                  */
+  float logit_scale;      /* logits = embed . norm(x) * logit_scale                                */
+} tgx_stack_desc;
+
 /* SamplerConfig (src/engine/Sampler.h:13-22).  Greedy iff temperature<=0 && top_k<=0 &&
  * top_p>=1 && min_p<=0 (Sampler.cpp:15-21). */
 typedef struct tgx_sampler_cfg {
@@ -108,6 +156,10 @@ TGX_API int tgx_device_count(int* out_count);
 /* == Model{Llama,Qwen2,Mistral}::Model*(config, device) (e.g. src/model/ModelLlama.h:57-65):
  * validates the description, binds the GPU, allocates parameter storage in compute_dtype. */
 TGX_API int tgx_create(const tgx_model_desc* desc, int device_ordinal, tgx_ctx** out_ctx);
+
+/* The layered counterpart of tgx_create: `layers` holds desc->layers entries.  Checkpoint names (tgx_upload): "embed", "final.norm",
+ * "l<i>.norm1|norm2|canon1|canon2|dwa", "l<i>.mix.q|dkv|dkv.norm|uk|uv|sink|g|o", "l<i>.mlp.router|router.b", "l<i>.mlp.e<j>.gate|up|down". */
+TGX_API int tgx_create_stack(const tgx_stack_desc* desc, const tgx_layer_desc* layers, int device_ordinal, tgx_ctx** out_ctx);
 
 /* == SafeTensors::loadInternal -> Storage::copyOnDevice for ONE named tensor
  * (src/util/SafeTensors.cpp:157-215).  `hf_name` is the checkpoint key; q/k/v and gate/up land in
@@ -191,6 +243,15 @@ TGX_API int tgx_reset_row(tgx_ctx* ctx, int row);
 TGX_API int tgx_forward_row(tgx_ctx* ctx, int row, const int64_t* ids, int seq);
 TGX_API int tgx_sample_row(tgx_ctx* ctx, int row, const tgx_sampler_cfg* cfg, uint64_t seed, int64_t* out_id);
 TGX_API int64_t tgx_past_length_row(const tgx_ctx* ctx, int row);
+
+/* One engine step over a RAGGED batch (layered models; the continuous-batching step the reference's README.md:33-34 leaves as a TODO): entry e
+ * brings counts[e] new tokens of slot rows[e] (distinct slots), all entries' ids concatenated in `ids`; each token attends its slot's cache
+ * and the tokens before it in the entry — portions of prompts and single decoded tokens share the pass.  A slot is admitted by its first
+ * entry (tgx_reset_row frees it) and may sit out any number of steps.  `want` lists n_want indices into the concatenated tokens whose logits are
+ * written to out_logits [n_want][vocab] (fp32, host).  When an entry's LAST token is wanted, its logits also become the slot's current logits
+ * (tgx_sample_row / tgx_read_logits).  Pages of the pool are assigned before anything is enqueued: TGX_ERR_CONTEXT leaves every slot as it was. */
+TGX_API int tgx_step_ragged(tgx_ctx* ctx, int n_entries, const int32_t* rows, const int32_t* counts, const int64_t* ids, int n_want,
+                            const int32_t* want, float* out_logits);
 
 /* == GPTModel::contextSize() / numLayers() (src/model/GPTModel.h:97-98). */
 TGX_API int64_t tgx_context_size(const tgx_ctx* ctx);

@@ -17,17 +17,19 @@ LIB = os.path.join(LIBDIR, "libtgx_mi355x.so")
 HIPCC = shutil.which("hipcc") or "/opt/rocm/bin/hipcc"
 FLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-shared", "-fvisibility=hidden",
          "-Wall", "-Wno-unused-function", "-DNDEBUG",
+         # no packed-fp32 VALU forms (v_pk_*_f32): scalar float code only
+         "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
          # MFMA accumulators in the (unified) VGPR file instead of AGPRs: the softmax / epilogue arithmetic reads them without
          # v_accvgpr_read/write copies (attention prefill: 127 of ~700 loop instructions) and most MFMA kernels need fewer registers
          ] + (["-mllvm", "-amdgpu-mfma-vgpr-form"] if os.environ.get("TGX_VGPR_FORM", "1") == "1" else [])
 
 
-TUS = ["abi", "decode", "attn", "sampler", "prefill", "prefill_f32", "skinny"]     # csrc/<name>.hip, compiled in parallel (csrc/ctx.h lists what each holds)
+TUS = ["abi", "decode", "attn", "sampler", "prefill", "prefill_f32", "skinny", "stack"]     # csrc/<name>.hip, compiled in parallel (csrc/ctx.h lists what each holds)
 OBJDIR = os.path.join(LIBDIR, "obj")
 
 
 def _deps():
-    deps = [os.path.join(HERE, "..", "include", "tgx.h"), os.path.join(CSRC, "ctx.h")]
+    deps = [os.path.join(HERE, "..", "include", "tgx.h"), os.path.join(CSRC, "ctx.h"), os.path.join(CSRC, "stack.h")]
     kd = os.path.join(CSRC, "kernels")
     return deps + [os.path.join(kd, f) for f in sorted(os.listdir(kd))]
 

@@ -6,6 +6,7 @@
 // There is NO CPU path in this library: every entry point either runs on the GPU or returns an error.
 #include <climits>
 #include "ctx.h"
+#include "stack.h"
 
 static std::string g_create_err;
 
@@ -171,6 +172,8 @@ void build_rope_host(const tgx_model_desc& d, std::vector<float>& cs, std::vecto
 }
 
 }  // namespace
+
+int upload_param_ext(tgx_ctx* c, ebyte* dst, const void* host, int64_t n, int src_dtype) { return upload_param(c, dst, host, n, src_dtype); }
 
 bool is_greedy(const tgx_sampler_cfg* s) {   // Sampler.cpp:15-21
   return !(s->temperature > 0.f || s->top_k > 0 || s->top_p < 1.f || s->min_p > 0.f);
@@ -503,9 +506,14 @@ int tgx_create(const tgx_model_desc* desc, int device_ordinal, tgx_ctx** out_ctx
   return TGX_OK;
 }
 
+int tgx_create_stack(const tgx_stack_desc* desc, const tgx_layer_desc* layers, int device_ordinal, tgx_ctx** out_ctx) {
+  return stack_create(desc, layers, device_ordinal, out_ctx);
+}
+
 int tgx_upload(tgx_ctx* c, const char* name, const void* host, const int64_t* shape, int nd, int src_dtype) {
   if (!c || !name || !host || !shape) return c ? set_err(c, TGX_ERR_INVALID, "null argument") : TGX_ERR_INVALID;
   HIP_OK(c, hipSetDevice(c->device));
+  if (c->stack) return stack_upload(c, name, host, shape, nd, src_dtype);
   const tgx_model_desc& d = c->d;
   const int64_t H = d.hidden, I = d.inter, V = d.vocab, qd = (int64_t)d.heads * d.head_dim, kvd = (int64_t)d.kv_heads * d.head_dim;
   auto bad_shape = [&]() { return set_err(c, TGX_ERR_SHAPE, "shape not equal for tensor: %s", name); };
@@ -578,6 +586,7 @@ int tgx_upload(tgx_ctx* c, const char* name, const void* host, const int64_t* sh
 int tgx_finalize(tgx_ctx* c) {
   if (!c) return TGX_ERR_INVALID;
   HIP_OK(c, hipSetDevice(c->device));
+  if (c->stack) return stack_finalize(c);
   const tgx_model_desc& d = c->d;
   const int H = d.hidden, I = d.inter, V = d.vocab, hd = d.head_dim, qd = d.heads * hd, kvd = d.kv_heads * hd;
   if (c->gpt2) {
@@ -709,6 +718,7 @@ void tgx_destroy(tgx_ctx* c) {
   (void)hipSetDevice(c->device);
   if (c->stream) (void)hipStreamSynchronize(c->stream);
   drop_step_graphs(c);
+  stack_destroy(c);
   auto fr = [](void* p) { if (p) (void)hipFree(p); };
   fr(c->embed); fr(c->lm_head); fr(c->final_norm); fr(c->wpe); fr(c->final_norm_b); fr(c->rope_cos); fr(c->rope_sin); fr(c->step); fr(c->step_done); fr(c->tok_log); fr(c->scratch_x); fr(c->seed_dev); fr(c->samp_scratch); fr(c->samp_list_comp); fr(c->samp_list_v);
   fr(c->slab_acc); fr(c->kv_tbl);
@@ -729,6 +739,12 @@ int tgx_forward(tgx_ctx* c, const int64_t* ids, int batch, int seq) {
   if (!c->finalized) return set_err(c, TGX_ERR_STATE, "forward before finalize");
   if (batch < 1 || batch > c->d.max_batch || seq < 1) return set_err(c, TGX_ERR_INVALID, "batch/seq out of range");
   if (c->poisoned) return set_err(c, TGX_ERR_STATE, "an earlier pass failed half-way: call tgx_reset_cache first");
+  if (c->stack) {      // a layered model: the rows' tokens as one ragged step (any pastLength per row), the last position's logits for every row
+    std::vector<int32_t> rws((size_t)batch), cnt((size_t)batch, seq), want((size_t)batch);
+    for (int b = 0; b < batch; b++) { rws[(size_t)b] = b; want[(size_t)b] = (b + 1) * seq - 1; }
+    std::vector<float> lg((size_t)batch * c->d.vocab);
+    return stack_step(c, batch, rws.data(), cnt.data(), ids, batch, want.data(), lg.data());
+  }
   if (seq > 1 && c->past > 0) return set_err(c, TGX_ERR_INVALID, "seq>1 with pastLength>0");
   if (c->past + seq > c->d.max_ctx) return set_err(c, TGX_ERR_CONTEXT, "context size exceeded: %lld + %d > %d", (long long)c->past, seq, c->d.max_ctx);
   for (int b = 0; b < batch; b++)
@@ -843,7 +859,7 @@ int tgx_decode(tgx_ctx* c, const tgx_sampler_cfg* cfg, uint64_t seed, int n_step
   if (n_steps > c->log_cap) return set_err(c, TGX_ERR_INVALID, "n_steps exceeds the token log capacity %d", c->log_cap);
   HIP_OK(c, hipSetDevice(c->device));
   const int64_t start = c->steps_issued;
-  int rc = run_decode_steps(c, *cfg, seed, n_steps);
+  int rc = c->stack ? stack_decode(c, *cfg, seed, n_steps) : run_decode_steps(c, *cfg, seed, n_steps);
   if (rc) return rc;
   c->have_logits = true;
   if (out_ids && n_steps > 0) {
@@ -867,7 +883,7 @@ int tgx_step_async(tgx_ctx* c, const tgx_sampler_cfg* cfg, uint64_t seed, int64_
   if (!c->have_token) return set_err(c, TGX_ERR_STATE, "step needs a current token: call tgx_sample after tgx_forward");
   if (c->past + 1 > c->d.max_ctx) return set_err(c, TGX_ERR_CONTEXT, "context size exceeded");
   HIP_OK(c, hipSetDevice(c->device));
-  int rc = run_decode_steps(c, *cfg, seed, 1);
+  int rc = c->stack ? stack_decode(c, *cfg, seed, 1) : run_decode_steps(c, *cfg, seed, 1);
   if (rc) return rc;
   const int64_t ticket = c->steps_issued;
   HIP_OK(c, hipEventRecord(c->ticket_ev[ticket % MAX_TICKET_EVENTS], c->stream));
@@ -890,6 +906,13 @@ int tgx_reset_cache(tgx_ctx* c) {
   if (!c) return TGX_ERR_INVALID;
   if (!c->finalized) return set_err(c, TGX_ERR_STATE, "reset before finalize");
   HIP_OK(c, hipSetDevice(c->device));
+  if (c->stack) {
+    for (int b = c->d.max_batch - 1; b >= 0; b--) { int rc = stack_reset_row(c, b); if (rc) return rc; }
+    c->batch = 0; c->past = 0;
+    std::fill(c->row_idle.begin(), c->row_idle.end(), 0);
+    c->have_logits = c->have_token = false;
+    return TGX_OK;
+  }
   for (auto& r : c->rows) HIP_OK(c, hipMemsetAsync(r.pos, 0, 4, c->stream));
   for (int b = 0; b < c->d.max_batch; b++) kv_release_row(c, b);
   if (c->slab_acc) HIP_OK(c, hipMemsetAsync(c->slab_acc, 0, (size_t)c->d.max_batch * c->d.hidden * 8, c->stream));
@@ -934,6 +957,7 @@ int tgx_reset_row(tgx_ctx* c, int row) {
   if (row < 0 || row >= c->d.max_batch) return set_err(c, TGX_ERR_INVALID, "row %d out of range [0,%d)", row, c->d.max_batch);
   if (c->poisoned) return set_err(c, TGX_ERR_STATE, "an earlier pass failed half-way: call tgx_reset_cache first");
   HIP_OK(c, hipSetDevice(c->device));
+  if (c->stack) return stack_reset_row(c, row);
   HIP_OK(c, hipMemsetAsync(c->rows[(size_t)row].pos, 0, 4, c->stream));     // stream-ordered behind the steps already enqueued
   kv_release_row(c, row);                                                     // paged KV: its blocks go back to the pool (a retired row rides along on the scratch block)
   c->row_past[(size_t)row] = 0;
@@ -947,6 +971,12 @@ int tgx_forward_row(tgx_ctx* c, int row, const int64_t* ids, int seq) {
   if (!c || !ids) return c ? set_err(c, TGX_ERR_INVALID, "null argument") : TGX_ERR_INVALID;
   if (!c->finalized) return set_err(c, TGX_ERR_STATE, "forward before finalize");
   if (c->poisoned) return set_err(c, TGX_ERR_STATE, "an earlier pass failed half-way: call tgx_reset_cache first");
+  if (c->stack) {      // a layered model: the next portion of the slot's sequence (its first admits it), logits of the portion's last token
+    const int32_t r = row, n = seq, w = seq - 1;
+    if (row < 0 || row >= c->d.max_batch || seq < 1) return set_err(c, TGX_ERR_INVALID, "row %d / seq %d out of range", row, seq);
+    std::vector<float> lg((size_t)c->d.vocab);
+    return stack_step(c, 1, &r, &n, ids, 1, &w, lg.data());
+  }
   if (row < 0 || row >= c->d.max_batch || row > c->batch) return set_err(c, TGX_ERR_INVALID, "row %d: a live row [0,%d) or the next free one (max_batch %d)", row, c->batch, c->d.max_batch);
   if (seq < 1 || seq > c->d.max_ctx) return set_err(c, seq < 1 ? TGX_ERR_INVALID : TGX_ERR_CONTEXT, "seq %d out of range (context size %d)", seq, c->d.max_ctx);
   if (!c->row_idle[(size_t)row] && c->row_past[(size_t)row] != 0) return set_err(c, TGX_ERR_STATE, "row %d holds %lld positions: tgx_reset_row first", row, (long long)c->row_past[(size_t)row]);
@@ -1045,7 +1075,15 @@ int tgx_synchronize(tgx_ctx* c) {
   return TGX_OK;
 }
 
+int tgx_step_ragged(tgx_ctx* c, int n_entries, const int32_t* rows, const int32_t* counts, const int64_t* ids, int n_want, const int32_t* want, float* out_logits) {
+  if (!c) return TGX_ERR_INVALID;
+  if (!c->stack) return set_err(c, TGX_ERR_UNSUPPORTED, "tgx_step_ragged serves layered models (tgx_create_stack); this family steps through tgx_forward_row / tgx_decode");
+  if (!c->finalized) return set_err(c, TGX_ERR_STATE, "step before finalize");
+  return stack_step(c, n_entries, rows, counts, ids, n_want, want, out_logits);
+}
+
 int tgx_read_kv(tgx_ctx* c, int row, int layer, float* k_out, float* v_out) {
+  if (c && c->stack) return c->finalized ? stack_read_latent(c, row, layer, k_out) : set_err(c, TGX_ERR_STATE, "read before finalize");      // the latent is all a layered model caches
   if (!c || !c->finalized || row < 0 || row >= c->d.max_batch || layer < 0 || layer >= c->d.layers) return TGX_ERR_INVALID;
   HIP_OK(c, hipSetDevice(c->device));
   HIP_OK(c, hipStreamSynchronize(c->stream));
@@ -1080,6 +1118,7 @@ int tgx_read_kv(tgx_ctx* c, int row, int layer, float* k_out, float* v_out) {
 }
 
 int tgx_write_kv(tgx_ctx* c, int row, int layer, const float* k_in, const float* v_in, int64_t n_rows) {
+  if (c && c->stack) return set_err(c, TGX_ERR_UNSUPPORTED, "tgx_write_kv: not provided for layered models");
   if (!c || !c->finalized || row < 0 || row >= c->d.max_batch || layer < 0 || layer >= c->d.layers || n_rows < 0 || n_rows > tgx_past_length_row(c, row)) return c ? set_err(c, TGX_ERR_INVALID, "write_kv: row / layer / n_rows out of range") : TGX_ERR_INVALID;
   HIP_OK(c, hipSetDevice(c->device));
   HIP_OK(c, hipStreamSynchronize(c->stream));
@@ -1113,6 +1152,7 @@ int tgx_write_kv(tgx_ctx* c, int row, int layer, const float* k_in, const float*
 }
 
 int tgx_profile_decode(tgx_ctx* c, int n_reps, int64_t* launches, double* total_ms) {
+  if (c && c->stack) return set_err(c, TGX_ERR_UNSUPPORTED, "tgx_profile_decode: not provided for layered models (their kernel times come from rocprofv3)");
   if (!c || !launches || !total_ms || n_reps < 0) return TGX_ERR_INVALID;
   if (!c->have_token) return set_err(c, TGX_ERR_STATE, "profile needs a current token: call tgx_sample after tgx_forward");
   if (c->past + 1 > c->d.max_ctx) return set_err(c, TGX_ERR_CONTEXT, "context size exceeded");
@@ -1182,6 +1222,13 @@ int tgx_set_logits(tgx_ctx* c, const float* logits, int batch) {
 
 int tgx_get_option(const tgx_ctx* c, const char* key, int* out_value) {
   if (!c || !key || !out_value) return TGX_ERR_INVALID;
+  if (c->stack) {
+    if (!strcmp(key, "kv.free_tokens")) { *out_value = stack_free_tokens(c); return TGX_OK; }
+    if (!strcmp(key, "kv.page_tokens")) { *out_value = c->stack->page; return TGX_OK; }
+    if (!strcmp(key, "act.round16")) { *out_value = c->act16; return TGX_OK; }
+    if (!strcmp(key, "attn.split_min")) { *out_value = c->stack->attn_split_min_keys; return TGX_OK; }
+    return TGX_ERR_INVALID;
+  }
   if (!strcmp(key, "attn.direct_limit")) { *out_value = (int)std::min<long long>(direct_limit(c, c->batch, true), INT_MAX); return TGX_OK; }
   if (!strcmp(key, "attn.nw4_limit")) { *out_value = (int)nw4_limit(c, c->batch, true); return TGX_OK; }
   if (!strcmp(key, "graph.steps")) { *out_value = c->graph_steps; return TGX_OK; }
@@ -1194,6 +1241,12 @@ int tgx_get_option(const tgx_ctx* c, const char* key, int* out_value) {
 int tgx_set_option(tgx_ctx* c, const char* key, int value) {
   if (!c || !key) return TGX_ERR_INVALID;
   static const char* cls_names[TGX_KERNEL_COUNT] = {"qkv", "attn", "oproj", "gateup", "down", "lmhead"};
+  if (c->stack) {      // layered models: "act.round16" as for the other families; "attn.split_min" = context from which steps of few tokens divide a sequence's keys
+    if (!strcmp(key, "act.round16")) { c->act16 = value != 0; return TGX_OK; }      // between workgroups; "stack.gemm_wt" forces the product tile (1 / 2, 0 = automatic)
+    if (!strcmp(key, "attn.split_min")) { c->stack->attn_split_min_keys = value; return TGX_OK; }
+    if (!strcmp(key, "stack.gemm_wt")) { if (value < 0 || value > 2) return set_err(c, TGX_ERR_INVALID, "stack.gemm_wt: 0, 1 or 2"); c->stack->gemm_wt = value; return TGX_OK; }
+    return set_err(c, TGX_ERR_INVALID, "unknown option %s for a layered model", key);
+  }
   drop_step_graphs(c);
   if (!strcmp(key, "graph")) { c->use_graph = value != 0; return TGX_OK; }
   if (!strcmp(key, "graph.steps")) { if (value < 1 || value > 64) return set_err(c, TGX_ERR_INVALID, "graph.steps out of range"); c->graph_steps = value; return TGX_OK; }
@@ -1285,6 +1338,7 @@ int tgx_set_option(tgx_ctx* c, const char* key, int value) {
 
 int64_t tgx_bytes_per_token(const tgx_ctx* c, int64_t T) {
   if (!c) return -1;
+  if (c->stack) return stack_bytes_per_token(c, T);
   const tgx_model_desc& d = c->d;
   const int64_t H = d.hidden, I = d.inter, V = d.vocab, L = d.layers, q = (int64_t)d.heads * d.head_dim, kv = (int64_t)d.kv_heads * d.head_dim;
   const int64_t b = (int64_t)c->esz;   // bytes per stored parameter / cache element

@@ -6,6 +6,7 @@
 //   prefill.hip      batched MFMA prefill, 16-bit storage (kernels/prefill.h, gemm_dma.h)
 //   prefill_f32.hip  batched prefill, fp32 storage (kernels/gemm_f32.h)
 //   skinny.hip       batched decode step / short prompts on the skinny MFMA GEMMs (kernels/skinny*.h)
+//   stack.hip        layered models (tgx_create_stack): ragged engine step, paged latent cache, slot state (kernels/stack*.h)
 // One context = one GPU = one HIP stream; every call comes from one host thread.  There is NO CPU path in this library.
 #pragma once
 #include <hip/hip_runtime.h>
@@ -26,6 +27,7 @@ using tgx::bf16_t;
 typedef unsigned char ebyte;   // parameter / KV-cache storage in the compute dtype: offsets are elements * ctx.esz
 
 namespace tgx { struct SampScratch; }
+struct StackModel;   // stack.h: a layered model (tgx_create_stack)
 
 constexpr int MAX_TICKET_EVENTS = 64;
 constexpr int HOST_RING = 256;
@@ -80,6 +82,7 @@ struct tgx_ctx {
   hipStream_t stream = nullptr;
   std::string err;
   bool finalized = false;
+  StackModel* stack = nullptr;   // set for layered models: the entry points of abi.hip hand over to stack.hip; `d` then carries hidden / layers / vocab / max_ctx / max_batch for the shared sampler
 
   int dt = tgx::DT_BF16;   // storage dtype of parameters and KV cache (kernel template argument)
   size_t esz = 2;          // bytes per stored element

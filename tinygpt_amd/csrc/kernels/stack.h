@@ -1,0 +1,337 @@
+// stack.h — the row-wise kernels of layered models (include/tgx.h tgx_stack_desc): every kernel works on the T tokens of one ragged engine step.
+// A step's tokens are the concatenated entries of its batch; StepMeta says which sequence slot and position each token belongs to.
+//   sinusoid_embed_kernel   embedding row + interleaved sin / cos position vector
+//   norm_conv_kernel        grouped RMS norm, the sublayer's causal short convolution over the normed rows, and the slot's convolution state
+//   latent_append_kernel    RMS norm of the down-projected latent and its store into the paged pool
+//   latent_attn_kernel      queries (already multiplied into latent space) against the pool: softmax with a sink, output in latent space
+//   latent_attn_split_kernel / latent_attn_merge_kernel   the same with a sequence's keys divided between workgroups (few tokens, long contexts)
+//   router_topk_kernel      32-bit router logits, top-k, softmax over the chosen
+//   moe_plan_kernel         (token, choice) pairs grouped by expert: offsets, permutation, tile list of the grouped products
+//   combine_depth_kernel    residual + weighted expert outputs, then the learned average over the embedding output and all layer results
+//   final_norm_rows_kernel  grouped RMS norm of the rows whose logits are asked for
+// All arithmetic here is fp32; reductions run in a fixed order.
+#pragma once
+#include "common.h"
+
+namespace tgx {
+
+struct StepMeta {          // device arrays of one step (T tokens, S entries)
+  const int* tok_id;       // [T] token id
+  const int* tok_pos;      // [T] position inside its sequence
+  const int* tok_ent;      // [T] entry of the token
+  const int* ent_row;      // [S] sequence slot
+  const int* ent_start;    // [S] first token of the entry
+  const int* ent_count;    // [S]
+  const int* ent_par;      // [S] which of the slot's two convolution-state buffers holds the state BEFORE this step
+  const int* tbl;          // [slots][tbl_stride] pages of the latent pool
+  int tbl_stride, page_shift, T, S;
+};
+
+// ---- x[t] = embed[id] + pe(pos): entry 2i = sin(pos * f_i), 2i + 1 = cos(pos * f_i); f (fp32) comes from the host.  Writes the stream and layer-result slot 0.
+template <int DT>
+__global__ __launch_bounds__(256) void sinusoid_embed_kernel(StepMeta m, const elem_t<DT>* embed, const float* freq, float* x, float* x0, int W) {
+  const int t = blockIdx.x;
+  const size_t id = (size_t)m.tok_id[t];
+  const float p = (float)m.tok_pos[t];
+  for (int c = threadIdx.x; c < W; c += 256) {
+    const float ang = p * freq[c >> 1];
+    const float pe = (c & 1) ? cosf(ang) : sinf(ang);
+    const float v = elem_to_f32<DT>(embed[id * W + c]) + pe;
+    x[(size_t)t * W + c] = v;
+    x0[(size_t)t * W + c] = v;
+  }
+}
+
+// ---- grouped RMS norm + input convolution.  One workgroup per token.  hn_r = x_r / rms_group(x_r) * w for the token and its taps - 1 predecessors
+// (rows of this step where the entry holds them, the slot's state otherwise, zero before the sequence's start);
+// out = hn_t + sum_j cw[:, j] * hn_(t - taps + 1 + j).  The state (the last taps - 1 normed rows of the slot) is double-buffered per slot: this
+// step reads buffer `par` and writes buffer `par ^ 1`, so no workgroup can overwrite what another still reads.
+constexpr int CONV_MAX_TAPS = 8, NORM_MAX_GROUPS = 16;
+struct NormConvArgs {
+  const float* x;        // [T][W]
+  const float* nw;       // [W] norm weight
+  const float* cw;       // [W][taps] convolution weight (nullptr: no convolution, taps = 1)
+  float* out;            // [T][W]
+  float* state;          // [2][slots][taps - 1][W] for this layer and sublayer (nullptr when taps == 1)
+  size_t state_buf;      // elements between the two buffers
+  int W, groups, taps;
+  float eps;
+};
+__global__ __launch_bounds__(256) void norm_conv_kernel(StepMeta m, NormConvArgs a) {
+  __shared__ float s_rinv[CONV_MAX_TAPS][NORM_MAX_GROUPS];
+  const int t = blockIdx.x, e = m.tok_ent[t], i = t - m.ent_start[e], cnt = m.ent_count[e], pos = m.tok_pos[t];
+  const int row = m.ent_row[e], par = m.ent_par[e];
+  const int lane = threadIdx.x & 63, wv = threadIdx.x >> 6;
+  const int gw = a.W / a.groups, nb = a.taps - 1;
+  // 1 / rms of every (row back, group) pair that lives in this step: one wave per pair, lanes over the group's channels
+  for (int it = wv; it < a.taps * a.groups; it += 4) {
+    const int d = it / a.groups, g = it - d * a.groups;
+    if (d > i) continue;                                  // wave-uniform: that row comes from the state (already normed) or lies before the start
+    const float* xr = a.x + (size_t)(t - d) * a.W + (size_t)g * gw;
+    float ss = 0.f;
+    for (int c = lane; c < gw; c += 64) ss = fmaf(xr[c], xr[c], ss);
+    ss = wave_sum(ss);
+    if (lane == 0) s_rinv[d][g] = 1.0f / sqrtf(ss / (float)gw + a.eps);
+  }
+  __syncthreads();
+  const float* st_old = a.state ? a.state + (size_t)par * a.state_buf + (size_t)row * nb * a.W : nullptr;
+  float* st_new = a.state ? a.state + (size_t)(par ^ 1) * a.state_buf + (size_t)row * nb * a.W : nullptr;
+  for (int c = threadIdx.x; c < a.W; c += 256) {
+    const int g = c / gw;
+    const float w = a.nw[c];
+    const float h0 = a.x[(size_t)t * a.W + c] * s_rinv[0][g] * w;
+    float acc = h0;
+    if (a.cw) {
+      acc = fmaf(a.cw[(size_t)c * a.taps + nb], h0, acc);
+      for (int d = 1; d <= nb; d++) {                      // the row d steps back
+        float hv = 0.f;
+        if (d <= i) hv = a.x[(size_t)(t - d) * a.W + c] * s_rinv[d][g] * w;
+        else if (pos - d >= 0) hv = st_old[(size_t)(nb - (d - i)) * a.W + c];       // state slot s holds position past - nb + s, past = pos - i
+        acc = fmaf(a.cw[(size_t)c * a.taps + (nb - d)], hv, acc);
+      }
+      // the slot's new state = the last nb normed rows after this step: row i of cnt lands in slot nb - (cnt - i) ...
+      const int s = nb - (cnt - i);
+      if (s >= 0) st_new[(size_t)s * a.W + c] = h0;
+      // ... and an entry shorter than the state keeps the tail of the old one (written by the entry's first token)
+      if (i == 0)
+        for (int k = 0; k + cnt < nb; k++) st_new[(size_t)k * a.W + c] = (pos - (nb - cnt - k) >= 0) ? st_old[(size_t)(k + cnt) * a.W + c] : 0.f;
+    }
+    a.out[(size_t)t * a.W + c] = acc;
+  }
+}
+
+// ---- latent: c = rms_norm(down-projected row) * w, stored at the token's place in the pool (storage dtype).  One wave per token.
+struct LatentAppendArgs {
+  const float* src; long long lds; int col0;     // the projection output [T][lds], latent columns from col0
+  const float* nw;                               // [rank]
+  void* pool;                                    // [pages][page][rank]
+  int rank; float eps;
+};
+template <int DT>
+__global__ __launch_bounds__(64) void latent_append_kernel(StepMeta m, LatentAppendArgs a) {
+  const int t = blockIdx.x, lane = threadIdx.x, e = m.tok_ent[t], pos = m.tok_pos[t];
+  const float* s = a.src + (size_t)t * a.lds + a.col0;
+  float ss = 0.f;
+  for (int c = lane; c < a.rank; c += 64) ss = fmaf(s[c], s[c], ss);
+  ss = wave_sum(ss);
+  const float rinv = 1.0f / sqrtf(ss / (float)a.rank + a.eps);
+  const int page = m.tbl[(size_t)m.ent_row[e] * m.tbl_stride + (pos >> m.page_shift)];
+  elem_t<DT>* dst = reinterpret_cast<elem_t<DT>*>(a.pool) + (((size_t)page << m.page_shift) + (size_t)(pos & ((1 << m.page_shift) - 1))) * a.rank;
+  for (int c = lane; c < a.rank; c += 64) dst[c] = f32_to_elem<DT>(s[c] * rinv * a.nw[c]);
+}
+
+// ---- latent attention, one workgroup per (token, head): the four waves take every fourth key, lanes hold rank / 64 latent channels each.
+// Scores are fp32 dot products of the latent-space query (score scale folded in) with the cached latents; the softmax denominator also holds
+// exp(sink[head]) — a term without key or value that counts once.  The output stays in latent space (the value up-projection follows as a product).
+constexpr int LAT_MAX_RPL = 16;       // latent channels per lane: rank <= 1024
+struct LatentAttnArgs {
+  const float* q; long long ldq;      // [T][heads * rank]
+  const void* pool;
+  const float* sink;                  // [heads]
+  float* out; long long ldo;          // [T][heads * rank]
+  int rank, heads;
+  // split form: keys [split * keys_per, ...) of every token's range; partial records (m, l, acc[rank]) per (token, head, split)
+  float* part; int nsplit, keys_per;
+};
+template <int DT, int RPL>
+__device__ __forceinline__ void latent_scan(const StepMeta& m, const LatentAttnArgs& a, int row, int j0, int j1, int jstep, const float* qv, float& mx, float& l, float* acc) {
+  const int lane = threadIdx.x & 63;
+  const elem_t<DT>* pool = reinterpret_cast<const elem_t<DT>*>(a.pool);
+  const int pmask = (1 << m.page_shift) - 1;
+  for (int j = j0; j < j1; j += jstep) {
+    const int page = m.tbl[(size_t)row * m.tbl_stride + (j >> m.page_shift)];
+    const elem_t<DT>* cr = pool + (((size_t)page << m.page_shift) + (size_t)(j & pmask)) * a.rank;
+    float cv[RPL];
+    float s = 0.f;
+#pragma unroll
+    for (int k = 0; k < RPL; k++) {
+      const int c = lane + 64 * k;
+      cv[k] = c < a.rank ? elem_to_f32<DT>(cr[c]) : 0.f;
+      s = fmaf(qv[k], cv[k], s);
+    }
+    s = wave_sum(s);
+    const float mn = fmaxf(mx, s);
+    const float corr = expf(mx - mn), p = expf(s - mn);      // mx = -inf on a wave's first key: corr = 0
+    l = fmaf(l, corr, p);
+#pragma unroll
+    for (int k = 0; k < RPL; k++) acc[k] = fmaf(acc[k], corr, p * cv[k]);
+    mx = mn;
+  }
+}
+template <int DT, int RPL, bool SPLIT>
+__global__ __launch_bounds__(256) void latent_attn_kernel(StepMeta m, LatentAttnArgs a) {
+  __shared__ float s_m[4], s_l[4];
+  extern __shared__ float s_acc[];      // [4][rank]
+  const int t = blockIdx.x, h = blockIdx.y, lane = threadIdx.x & 63, wv = threadIdx.x >> 6;
+  const int row = m.ent_row[m.tok_ent[t]], nkeys = m.tok_pos[t] + 1;
+  int k0 = 0, k1 = nkeys;
+  if (SPLIT) { k0 = min(nkeys, (int)blockIdx.z * a.keys_per); k1 = min(nkeys, k0 + a.keys_per); }
+  const float* q = a.q + (size_t)t * a.ldq + (size_t)h * a.rank;
+  float qv[RPL], acc[RPL];
+#pragma unroll
+  for (int k = 0; k < RPL; k++) { const int c = lane + 64 * k; qv[k] = c < a.rank ? q[c] : 0.f; acc[k] = 0.f; }
+  // the sink enters once: as the starting state of wave 0 (of split 0)
+  const bool has_sink = wv == 0 && (!SPLIT || blockIdx.z == 0);
+  float mx = has_sink ? a.sink[h] : -INFINITY, l = has_sink ? 1.f : 0.f;
+  latent_scan<DT, RPL>(m, a, row, k0 + wv, k1, 4, qv, mx, l, acc);
+  if (lane == 0) { s_m[wv] = mx; s_l[wv] = l; }
+#pragma unroll
+  for (int k = 0; k < RPL; k++) { const int c = lane + 64 * k; if (c < a.rank) s_acc[wv * a.rank + c] = acc[k]; }
+  __syncthreads();
+  const float M = fmaxf(fmaxf(s_m[0], s_m[1]), fmaxf(s_m[2], s_m[3]));
+  float f[4], L = 0.f;
+#pragma unroll
+  for (int w = 0; w < 4; w++) { f[w] = s_m[w] == -INFINITY ? 0.f : expf(s_m[w] - M); L = fmaf(s_l[w], f[w], L); }
+  if (SPLIT) {
+    float* rec = a.part + (((size_t)t * a.heads + h) * a.nsplit + blockIdx.z) * (size_t)(a.rank + 2);
+    if (threadIdx.x == 0) { rec[0] = M; rec[1] = L; }
+    for (int c = threadIdx.x; c < a.rank; c += 256) rec[2 + c] = s_acc[c] * f[0] + s_acc[a.rank + c] * f[1] + s_acc[2 * a.rank + c] * f[2] + s_acc[3 * a.rank + c] * f[3];
+  } else {
+    const float inv = 1.0f / L;
+    float* o = a.out + (size_t)t * a.ldo + (size_t)h * a.rank;
+    for (int c = threadIdx.x; c < a.rank; c += 256) o[c] = (s_acc[c] * f[0] + s_acc[a.rank + c] * f[1] + s_acc[2 * a.rank + c] * f[2] + s_acc[3 * a.rank + c] * f[3]) * inv;
+  }
+}
+// merges the split records of one (token, head) in split order
+__global__ __launch_bounds__(256) void latent_attn_merge_kernel(LatentAttnArgs a) {
+  const int t = blockIdx.x, h = blockIdx.y;
+  const float* rec = a.part + ((size_t)t * a.heads + h) * a.nsplit * (size_t)(a.rank + 2);
+  float M = -INFINITY;
+  for (int s = 0; s < a.nsplit; s++) M = fmaxf(M, rec[(size_t)s * (a.rank + 2)]);
+  float L = 0.f;
+  for (int s = 0; s < a.nsplit; s++) { const float ms = rec[(size_t)s * (a.rank + 2)]; L = fmaf(rec[(size_t)s * (a.rank + 2) + 1], ms == -INFINITY ? 0.f : expf(ms - M), L); }
+  const float inv = 1.0f / L;
+  float* o = a.out + (size_t)t * a.ldo + (size_t)h * a.rank;
+  for (int c = threadIdx.x; c < a.rank; c += 256) {
+    float v = 0.f;
+    for (int s = 0; s < a.nsplit; s++) { const float ms = rec[(size_t)s * (a.rank + 2)]; v = fmaf(rec[(size_t)s * (a.rank + 2) + 2 + c], ms == -INFINITY ? 0.f : expf(ms - M), v); }
+    o[c] = v * inv;
+  }
+}
+
+// ---- router: z = Wr h + b in fp32 (one wave per expert, lanes over the width), the `top` largest (ties: the lower index), weights = softmax over them
+struct RouterArgs {
+  const float* h;        // [T][W]
+  const float* wr;       // [E][W] fp32
+  const float* br;       // [E]
+  int* sel;              // [T][top]
+  float* selw;           // [T][top]
+  int W, E, top;
+};
+constexpr int ROUTER_MAX_E = 1024, ROUTER_MAX_TOP = 64;
+__global__ __launch_bounds__(256) void router_topk_kernel(RouterArgs a) {
+  __shared__ float s_z[ROUTER_MAX_E];
+  __shared__ float s_v[ROUTER_MAX_TOP];
+  __shared__ int s_i[ROUTER_MAX_TOP];
+  const int t = blockIdx.x, lane = threadIdx.x & 63, wv = threadIdx.x >> 6;
+  const float* h = a.h + (size_t)t * a.W;
+  for (int e = wv; e < a.E; e += 4) {
+    const float* w = a.wr + (size_t)e * a.W;
+    float s = 0.f;
+    for (int c = lane; c < a.W; c += 64) s = fmaf(h[c], w[c], s);
+    s = wave_sum(s);
+    if (lane == 0) s_z[e] = s + a.br[e];
+  }
+  __syncthreads();
+  if (wv == 0) {
+    // every lane owns the logits e = lane, lane + 64, ...: it alone reads and retires them, so the loop needs no barrier; the butterfly leaves each
+    // pick in all lanes, lane 0 keeps the list
+    for (int k = 0; k < a.top; k++) {
+      float bv = -INFINITY; int bi = 0x7fffffff;
+      for (int e = lane; e < a.E; e += 64) { const float v = s_z[e]; if (v > bv) { bv = v; bi = e; } }
+      for (int o = 32; o > 0; o >>= 1) {
+        const float ov = __shfl_xor(bv, o, 64); const int oi = __shfl_xor(bi, o, 64);
+        if (ov > bv || (ov == bv && oi < bi)) { bv = ov; bi = oi; }
+      }
+      if (bi < a.E && (bi & 63) == lane) s_z[bi] = -INFINITY;
+      if (lane == 0) { s_v[k] = bv; s_i[k] = bi < a.E ? bi : 0; }
+    }
+    if (lane == 0) {
+      const float mx = s_v[0];            // the first pick is the largest
+      float den = 0.f;
+      for (int k = 0; k < a.top; k++) den += expf(s_v[k] - mx);
+      for (int k = 0; k < a.top; k++) { a.sel[(size_t)t * a.top + k] = s_i[k]; a.selw[(size_t)t * a.top + k] = expf(s_v[k] - mx) / den; }
+    }
+  }
+}
+
+// ---- plan of the grouped expert products: pairs i = t * top + k grouped by expert.  One workgroup.
+//   off[E + 1]   first grouped row of every expert;  perm[n]  the pair at grouped row n;  tok[n] = perm[n] / top (the row of the activations)
+//   tiles: (expert, first row) of every tile of tile_m rows, n_tiles of them
+struct MoePlanArgs {
+  const int* sel; int n_pairs, E, top, tile_m;
+  int *off, *perm, *tok, *tile_e, *tile_m0, *n_tiles;
+};
+__global__ __launch_bounds__(1024) void moe_plan_kernel(MoePlanArgs a) {
+  __shared__ int s_cnt[ROUTER_MAX_E], s_off[ROUTER_MAX_E + 1], s_cur[ROUTER_MAX_E];
+  for (int e = threadIdx.x; e < a.E; e += 1024) { s_cnt[e] = 0; s_cur[e] = 0; }
+  __syncthreads();
+  for (int i = threadIdx.x; i < a.n_pairs; i += 1024) atomicAdd(&s_cnt[a.sel[i]], 1);
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    int o = 0, nt = 0;
+    for (int e = 0; e < a.E; e++) {
+      s_off[e] = o; a.off[e] = o;
+      for (int m0 = 0; m0 < s_cnt[e]; m0 += a.tile_m) { a.tile_e[nt] = e; a.tile_m0[nt] = o + m0; nt++; }
+      o += s_cnt[e];
+    }
+    s_off[a.E] = o; a.off[a.E] = o;
+    *a.n_tiles = nt;
+  }
+  __syncthreads();
+  // rows of an expert in any order: every pair's result lands in its own output row, so the order changes no value
+  for (int i = threadIdx.x; i < a.n_pairs; i += 1024) {
+    const int e = a.sel[i];
+    const int n = s_off[e] + atomicAdd(&s_cur[e], 1);
+    a.perm[n] = i; a.tok[n] = i / a.top;
+  }
+}
+
+// ---- x_new = x + sum_k y[t * top + k] (router weights already applied), stored as the layer's result X_(i+1); the stream handed on is
+// sum_j dw[j] X_j over the embedding output and all results so far.
+struct CombineDepthArgs {
+  float* x;              // [T][W] in: the stream after the mixer; out: the next layer's input
+  const float* y;        // [T * top][W] expert outputs (nullptr / top 0: no feed-forward)
+  float* xs;             // [n_res][slot_stride] layer results; this layer writes slot n_res - 1
+  size_t slot_stride;
+  const float* dw;       // [n_res]
+  int W, top, n_res;
+};
+__global__ __launch_bounds__(256) void combine_depth_kernel(CombineDepthArgs a) {
+  const size_t t = blockIdx.x;
+  for (int c = threadIdx.x; c < a.W; c += 256) {
+    float v = a.x[t * a.W + c];
+    for (int k = 0; k < a.top; k++) v += a.y[(t * a.top + k) * a.W + c];
+    a.xs[(size_t)(a.n_res - 1) * a.slot_stride + t * a.W + c] = v;
+    float s = 0.f;
+    for (int j = 0; j < a.n_res - 1; j++) s = fmaf(a.dw[j], a.xs[(size_t)j * a.slot_stride + t * a.W + c], s);
+    a.x[t * a.W + c] = fmaf(a.dw[a.n_res - 1], v, s);
+  }
+}
+
+// ---- out[i] = grouped RMS norm of x[rows[i]] * w
+__global__ __launch_bounds__(256) void final_norm_rows_kernel(const float* x, const int* rows, const float* nw, float* out, int W, int groups, float eps) {
+  __shared__ float s_rinv[NORM_MAX_GROUPS];
+  const int lane = threadIdx.x & 63, wv = threadIdx.x >> 6, gw = W / groups;
+  const float* xr = x + (size_t)rows[blockIdx.x] * W;
+  for (int g = wv; g < groups; g += 4) {
+    float ss = 0.f;
+    for (int c = lane; c < gw; c += 64) ss = fmaf(xr[(size_t)g * gw + c], xr[(size_t)g * gw + c], ss);
+    ss = wave_sum(ss);
+    if (lane == 0) s_rinv[g] = 1.0f / sqrtf(ss / (float)gw + eps);
+  }
+  __syncthreads();
+  for (int c = threadIdx.x; c < W; c += 256) out[(size_t)blockIdx.x * W + c] = xr[c] * s_rinv[c / gw] * nw[c];
+}
+
+// decode steps: the tokens come from the slots' device-resident current tokens, and positions advance on the device
+__global__ void stack_gather_tok_kernel(int* tok_id, const int* ent_row, const int* slab_tok, int S) {
+  const int i = blockIdx.x * blockDim.x + threadIdx.x;
+  if (i < S) tok_id[i] = slab_tok[ent_row[i]];
+}
+__global__ void stack_advance_kernel(int* tok_pos, int* ent_par, int S) {
+  const int i = blockIdx.x * blockDim.x + threadIdx.x;
+  if (i < S) { tok_pos[i] += 1; ent_par[i] ^= 1; }
+}
+
+}  // namespace tgx

@@ -1,0 +1,235 @@
+// stack_gemm.h — the matrix products of layered models: C = epilogue(A · Bᵀ) with fp32 activations A [M][K] and stored weights B [N][K].
+//   16-bit storage: v_mfma_f32_32x32x16 on the activation's two 16-bit terms (x = hi + lo, 16 significant bits) — or its rounded first term alone
+//   (option act.round16) — against the stored weight, fp32 accumulation; fp32 storage: v_mfma_f32_32x32x2_f32, nothing rounded.
+// One kernel serves plain, batched and grouped products:
+//   batched (blockIdx.z = head):   B advances by b_zstride, the A / C columns by a_zoff / c_zoff per z — per-head products on slices of wide rows
+//   grouped (experts):             blockIdx.y walks a tile list (expert, first row) built on the device (moe_plan_kernel); rows are gathered through
+//                                  a_rows and scattered through c_rows
+//   dual:                          two weight matrices against the same activation tile (an expert's gate and up projections), combined in the epilogue
+// Workgroup = 4 waves as 2 x 2, each WT x WT tiles of 32 x 32: 64 WT x 64 WT outputs per workgroup, K in steps of 32 staged through LDS with the
+// next step's global loads in flight under the MFMAs.  Any M, N, K: rows, columns and the K tail are masked; shapes that break the 16-byte
+// alignment of the vector loads take element loads (VEC = false).
+#pragma once
+#include "prefill.h"
+
+namespace tgx {
+
+enum { SG_STORE = 0, SG_ADD = 1, SG_GATE = 2, SG_EXPERT_ACT = 3, SG_ROWSCALE = 4 };
+struct StackGemmArgs {
+  const float* A; long long lda; int a_zoff;
+  const int* a_rows;
+  const void* B; const void* B2; long long ldb; long long b_zstride;
+  float* C; long long ldc; int c_zoff;
+  const int* c_rows;
+  const int* z_off; const int* tile_z; const int* tile_m0; const int* n_tiles;      // grouped
+  int M, N, K;
+  float scale;                 // SG_STORE: C = acc * scale
+  float limit;                 // SG_EXPERT_ACT
+  const float* G; long long ldg; int g_col0;     // SG_GATE: C = acc * sigmoid(G[row][g_col0 + z * c_zoff + n])
+  const float* rw;             // SG_ROWSCALE: C = acc * rw[c row]
+  int terms;                   // 16-bit storage: 2 = hi + lo, 1 = hi only
+};
+
+// an expert's activation: g = min(gate, limit), u = clamp(up, -limit, limit); g * sigmoid(1.702 g) * (u + 1)
+__device__ __forceinline__ float expert_act(float gate, float up, float limit) {
+  const float g = fminf(gate, limit), u = fminf(fmaxf(up, -limit), limit);
+  return g / (1.0f + expf(-1.702f * g)) * (u + 1.0f);
+}
+
+template <int DT, int EPI, bool DUAL, int WT, bool VEC>
+__global__ __launch_bounds__(256) void stack_gemm_kernel(const StackGemmArgs a) {
+  constexpr int BM = 64 * WT, BN = 64 * WT, BK = 32;
+  constexpr bool F32 = DT == DT_F32;
+  constexpr int LDK = BK + 8;                       // 16-bit tiles: row-major, k contiguous, 16 bytes of padding
+  constexpr int LDA = BM + 1, LDB = BN + 1;         // fp32 tiles: k-major
+  constexpr int NB = DUAL ? 2 : 1;
+  extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
+  bf16_t* sAh = reinterpret_cast<bf16_t*>(smem);
+  bf16_t* sAl = sAh + BM * LDK;
+  bf16_t* sB = sAl + BM * LDK;                      // [NB][BN][LDK]
+  float* fA = reinterpret_cast<float*>(smem);       // [BK][LDA]
+  float* fB = fA + BK * LDA;                        // [NB][BK][LDB]
+
+  const int tid = threadIdx.x, lane = tid & 63, wv = tid >> 6, wm = wv >> 1, wn = wv & 1;
+  int z, mbase, mend;
+  if (a.z_off) {
+    if ((int)blockIdx.y >= *a.n_tiles) return;
+    z = a.tile_z[blockIdx.y]; mbase = a.tile_m0[blockIdx.y]; mend = a.z_off[z + 1];
+  } else { z = blockIdx.z; mbase = blockIdx.y * BM; mend = a.M; }
+  const int n0 = blockIdx.x * BN;
+  const float* Ab = a.A + (size_t)z * a.a_zoff;
+  const elem_t<DT>* Bz[NB];
+  Bz[0] = reinterpret_cast<const elem_t<DT>*>(a.B) + (size_t)z * a.b_zstride;
+  if constexpr (DUAL) Bz[1] = reinterpret_cast<const elem_t<DT>*>(a.B2) + (size_t)z * a.b_zstride;
+
+  f32x16 acc[NB][WT][WT];
+#pragma unroll
+  for (int b = 0; b < NB; b++)
+#pragma unroll
+    for (int i = 0; i < WT; i++)
+#pragma unroll
+      for (int j = 0; j < WT; j++)
+#pragma unroll
+        for (int r = 0; r < 16; r++) acc[b][i][j][r] = 0.f;
+
+  // ---- staging maps.  A: chunks of 4 k (fp32) -> chunk c: row c / 8, k 4 (c % 8).  B: 16-bit chunks of 8 k -> row c / 4, k 8 (c % 4); fp32 as A.
+  constexpr int AI = BM * (BK / 4) / 256;
+  constexpr int BI = F32 ? BN * (BK / 4) / 256 : BN * (BK / 8) / 256;
+  f32x4 ra[AI];
+  f32x4 rbf[F32 ? NB * BI : 1];
+  u32x4 rbh[F32 ? 1 : NB * BI];
+  size_t arow[AI];
+#pragma unroll
+  for (int i = 0; i < AI; i++) {
+    const int m = mbase + (tid + 256 * i) / 8;
+    const int mc = min(m, mend - 1);
+    arow[i] = (size_t)(a.a_rows ? a.a_rows[mc] : mc) * a.lda;
+  }
+  auto load_tiles = [&](int k0) {
+#pragma unroll
+    for (int i = 0; i < AI; i++) {
+      const int k = k0 + 4 * ((tid + 256 * i) & 7);
+      const float* p = Ab + arow[i] + k;
+      if (VEC) ra[i] = k < a.K ? *reinterpret_cast<const f32x4*>(p) : f32x4{0.f, 0.f, 0.f, 0.f};
+      else
+#pragma unroll
+        for (int e = 0; e < 4; e++) ra[i][e] = k + e < a.K ? p[e] : 0.f;
+    }
+#pragma unroll
+    for (int b = 0; b < NB; b++)
+#pragma unroll
+      for (int i = 0; i < BI; i++) {
+        const int c = tid + 256 * i;
+        if constexpr (F32) {
+          const int n = min(n0 + c / 8, a.N - 1), k = k0 + 4 * (c & 7);
+          const float* p = reinterpret_cast<const float*>(Bz[b]) + (size_t)n * a.ldb + k;
+          if (VEC) rbf[b * BI + i] = k < a.K ? *reinterpret_cast<const f32x4*>(p) : f32x4{0.f, 0.f, 0.f, 0.f};
+          else
+#pragma unroll
+            for (int e = 0; e < 4; e++) rbf[b * BI + i][e] = k + e < a.K ? p[e] : 0.f;
+        } else {
+          const int n = min(n0 + c / 4, a.N - 1), k = k0 + 8 * (c & 3);
+          const bf16_t* p = reinterpret_cast<const bf16_t*>(Bz[b]) + (size_t)n * a.ldb + k;
+          if (VEC) rbh[b * BI + i] = k < a.K ? *reinterpret_cast<const u32x4*>(p) : u32x4{0u, 0u, 0u, 0u};
+          else {
+            u32x4 v = {0u, 0u, 0u, 0u};
+#pragma unroll
+            for (int e = 0; e < 8; e++) if (k + e < a.K) v[e >> 1] |= (unsigned int)p[e] << (16 * (e & 1));
+            rbh[b * BI + i] = v;
+          }
+        }
+      }
+  };
+  auto store_tiles = [&]() {
+#pragma unroll
+    for (int i = 0; i < AI; i++) {
+      const int c = tid + 256 * i, row = c / 8, kc = c & 7;
+      if constexpr (F32) {
+#pragma unroll
+        for (int e = 0; e < 4; e++) fA[(4 * kc + e) * LDA + row] = ra[i][e];
+      } else {
+        bf16_t h[4], l[4];
+#pragma unroll
+        for (int e = 0; e < 4; e++) split16<DT>(ra[i][e], h[e], l[e]);
+        *reinterpret_cast<u32x2*>(sAh + row * LDK + 4 * kc) = u32x2{(unsigned int)h[0] | ((unsigned int)h[1] << 16), (unsigned int)h[2] | ((unsigned int)h[3] << 16)};
+        *reinterpret_cast<u32x2*>(sAl + row * LDK + 4 * kc) = u32x2{(unsigned int)l[0] | ((unsigned int)l[1] << 16), (unsigned int)l[2] | ((unsigned int)l[3] << 16)};
+      }
+    }
+#pragma unroll
+    for (int b = 0; b < NB; b++)
+#pragma unroll
+      for (int i = 0; i < BI; i++) {
+        const int c = tid + 256 * i;
+        if constexpr (F32) {
+          const int row = c / 8, kc = c & 7;
+#pragma unroll
+          for (int e = 0; e < 4; e++) fB[(b * BK + 4 * kc + e) * LDB + row] = rbf[b * BI + i][e];
+        } else {
+          const int row = c / 4, kc = c & 3;
+          *reinterpret_cast<u32x4*>(sB + ((size_t)b * BN + row) * LDK + 8 * kc) = rbh[b * BI + i];
+        }
+      }
+  };
+
+  load_tiles(0);
+  for (int k0 = 0; k0 < a.K; k0 += BK) {
+    __syncthreads();
+    store_tiles();
+    __syncthreads();
+    if (k0 + BK < a.K) load_tiles(k0 + BK);
+    if constexpr (F32) {
+#pragma unroll
+      for (int kk = 0; kk < BK / 2; kk++) {
+        const int krow = 2 * kk + (lane >> 5);
+        float fa[WT], fb[NB][WT];
+#pragma unroll
+        for (int i = 0; i < WT; i++) fa[i] = fA[krow * LDA + wm * (32 * WT) + i * 32 + (lane & 31)];
+#pragma unroll
+        for (int b = 0; b < NB; b++)
+#pragma unroll
+          for (int j = 0; j < WT; j++) fb[b][j] = fB[(b * BK + krow) * LDB + wn * (32 * WT) + j * 32 + (lane & 31)];
+#pragma unroll
+        for (int b = 0; b < NB; b++)
+#pragma unroll
+          for (int i = 0; i < WT; i++)
+#pragma unroll
+            for (int j = 0; j < WT; j++) acc[b][i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(fa[i], fb[b][j], acc[b][i][j], 0, 0, 0);
+      }
+    } else {
+#pragma unroll
+      for (int kk = 0; kk < BK / 16; kk++) {
+        const int kof = 16 * kk + 8 * (lane >> 5);
+        bf16x8 ah[WT], al[WT], bb[NB][WT];
+#pragma unroll
+        for (int i = 0; i < WT; i++) {
+          const int row = wm * (32 * WT) + i * 32 + (lane & 31);
+          ah[i] = *reinterpret_cast<const bf16x8*>(sAh + row * LDK + kof);
+          al[i] = *reinterpret_cast<const bf16x8*>(sAl + row * LDK + kof);
+        }
+#pragma unroll
+        for (int b = 0; b < NB; b++)
+#pragma unroll
+          for (int j = 0; j < WT; j++) bb[b][j] = *reinterpret_cast<const bf16x8*>(sB + ((size_t)b * BN + wn * (32 * WT) + j * 32 + (lane & 31)) * LDK + kof);
+#pragma unroll
+        for (int b = 0; b < NB; b++)
+#pragma unroll
+          for (int i = 0; i < WT; i++)
+#pragma unroll
+            for (int j = 0; j < WT; j++) {
+              acc[b][i][j] = mfma16<DT>(ah[i], bb[b][j], acc[b][i][j]);
+              if (a.terms > 1) acc[b][i][j] = mfma16<DT>(al[i], bb[b][j], acc[b][i][j]);
+            }
+      }
+    }
+  }
+
+  // ---- epilogue.  C / D layout of the 32 x 32 product: column = lane & 31, row = (r & 3) + 8 (r >> 2) + 4 (lane >> 5)
+#pragma unroll
+  for (int i = 0; i < WT; i++)
+#pragma unroll
+    for (int r = 0; r < 16; r++) {
+      const int m = mbase + wm * (32 * WT) + i * 32 + (r & 3) + 8 * (r >> 2) + 4 * (lane >> 5);
+      if (m >= mend) continue;
+      const size_t crow = a.c_rows ? (size_t)a.c_rows[m] : (size_t)m;
+      float* cp = a.C + crow * a.ldc + (size_t)z * a.c_zoff;
+#pragma unroll
+      for (int j = 0; j < WT; j++) {
+        const int n = n0 + wn * (32 * WT) + j * 32 + (lane & 31);
+        if (n >= a.N) continue;
+        const float v = acc[0][i][j][r];
+        if constexpr (EPI == SG_STORE) cp[n] = v * a.scale;
+        else if constexpr (EPI == SG_ADD) cp[n] += v;
+        else if constexpr (EPI == SG_GATE) cp[n] = v / (1.0f + expf(-a.G[crow * a.ldg + a.g_col0 + (size_t)z * a.c_zoff + n]));
+        else if constexpr (EPI == SG_EXPERT_ACT) cp[n] = expert_act(v, acc[NB - 1][i][j][r], a.limit);
+        else cp[n] = v * a.rw[crow];
+      }
+    }
+}
+
+template <int DT, bool DUAL, int WT>
+constexpr size_t stack_gemm_lds() {
+  constexpr int BM = 64 * WT, BN = 64 * WT, BK = 32, NB = DUAL ? 2 : 1;
+  return DT == DT_F32 ? (size_t)(BK * (BM + 1) + NB * BK * (BN + 1)) * 4 : (size_t)(2 * BM + NB * BN) * (BK + 8) * 2;
+}
+
+}  // namespace tgx

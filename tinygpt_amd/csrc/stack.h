@@ -1,0 +1,59 @@
+// stack.h — host-side state of a layered model (include/tgx.h tgx_stack_desc): per-layer weights, the paged latent pool with its page tables,
+// the slots' convolution state and the workspace of one ragged step.  Owned by tgx_ctx::stack; the launch code lives in stack.hip.
+#pragma once
+#include <set>
+#include <string>
+#include <vector>
+
+#include "ctx.h"
+
+struct StackLayerW {
+  tgx_layer_desc d{};
+  float *norm1 = nullptr, *norm2 = nullptr, *canon1 = nullptr, *canon2 = nullptr, *dwa = nullptr;      // fp32
+  // mixer (latent attention)
+  ebyte* w_in = nullptr;        // [heads * dim | kv_rank | heads * vdim][width]: query, latent and gate projections in one product
+  ebyte* w_ukT = nullptr;       // [heads][kv_rank][dim]: the key up-projection, transposed per head (queries are multiplied into latent space)
+  ebyte* w_uv = nullptr;        // [heads * vdim][kv_rank]
+  ebyte* w_o = nullptr;         // [width][heads * vdim]
+  float *lat_norm = nullptr, *sink = nullptr;
+  // feed-forward (mixture of experts)
+  ebyte *w_gate = nullptr, *w_up = nullptr, *w_down = nullptr;      // [experts][ff][width] x 2, [experts][width][ff]
+  float *w_router = nullptr, *b_router = nullptr;                   // fp32 [experts][width], [experts]
+  ebyte* pool = nullptr;        // latent cache of this layer: [pages][page_tokens][kv_rank]
+  float* conv_state = nullptr;  // [2 sublayers][2 buffers][slots][taps - 1][width]
+};
+
+struct StackModel {
+  tgx_stack_desc d{};
+  std::vector<StackLayerW> L;
+  std::set<std::string> missing;       // checkpoint names not uploaded yet
+  float *final_norm = nullptr, *freq = nullptr;
+  // pages
+  int page = 64, page_shift = 6, n_pages = 0, tbl_stride = 0;
+  int* tbl_dev = nullptr;
+  int* tbl_host = nullptr;             // pinned mirror [slots][tbl_stride]
+  std::vector<int> free_pages, row_pages, row_par;
+  std::vector<char> row_dirty;
+  // step workspace, grown to the largest step seen
+  int cap_tokens = 0, cap_want = 0;
+  int* meta_dev = nullptr; int* meta_host = nullptr; size_t meta_cap = 0;      // one block of ints: the StepMeta arrays + the wanted rows
+  hipEvent_t meta_ev = nullptr; bool meta_pending = false;
+  float *x = nullptr, *xs = nullptr, *a = nullptr, *proj = nullptr, *ql = nullptr, *lat = nullptr, *o = nullptr;
+  float *selw = nullptr, *yh = nullptr, *yd = nullptr, *xn = nullptr, *lg = nullptr, *part = nullptr;
+  size_t part_elems = 0;
+  int *sel = nullptr, *moe_off = nullptr, *perm = nullptr, *ptok = nullptr, *tile_e = nullptr, *tile_m0 = nullptr, *n_tiles = nullptr;
+  int max_in = 0, max_hr = 0, max_hv = 0, max_top = 0, max_ff = 0, max_E = 0, max_rank = 0;
+  int attn_split_min_keys = 2048;      // option attn.split_min: steps of few tokens split a sequence's keys between workgroups from this context on
+  int gemm_wt = 0;                     // option stack.gemm_wt: force the product's tile (1: 64 x 64, 2: 128 x 128); 0 = by the number of tiles
+};
+
+int stack_create(const tgx_stack_desc* desc, const tgx_layer_desc* layers, int device_ordinal, tgx_ctx** out_ctx);
+int stack_upload(tgx_ctx* c, const char* name, const void* host, const int64_t* shape, int nd, int src_dtype);
+int stack_finalize(tgx_ctx* c);
+void stack_destroy(tgx_ctx* c);
+int stack_step(tgx_ctx* c, int n_entries, const int32_t* rows, const int32_t* counts, const int64_t* ids, int n_want, const int32_t* want, float* out_logits);
+int stack_decode(tgx_ctx* c, const tgx_sampler_cfg& cfg, uint64_t seed, int n_steps);
+int stack_reset_row(tgx_ctx* c, int row);
+int stack_free_tokens(const tgx_ctx* c);
+int stack_read_latent(tgx_ctx* c, int row, int layer, float* out);
+int64_t stack_bytes_per_token(const tgx_ctx* c, int64_t T);

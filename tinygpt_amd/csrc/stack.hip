@@ -1,0 +1,679 @@
+// stack.hip — layered models behind the C ABI (include/tgx.h tgx_create_stack / tgx_step_ragged): creation from a per-layer description, weight upload by
+// checkpoint name, the paged latent pool and the slots' convolution state, the ragged engine step, and the decode loop on top of the shared sampler.
+//
+// One step = T tokens of S entries (a portion of a prompt, or one decoded token, per sequence slot).  Per layer:
+//   norm_conv (norm1, canon1) -> one product for [queries | latent | gate] -> latent norm + pool append -> queries into latent space (per head)
+//   -> latent attention over the pool -> value up-projection with the sigmoid gate in its epilogue -> output product added to the stream
+//   -> norm_conv (norm2, canon2) -> router top-k -> grouped expert products (gate / up with the activation, down with the router weight)
+//   -> combine + depth average.
+// Attention reads every key from the pool — also the keys of the step's own tokens, appended before it runs — so a position's result does not depend
+// on how its sequence was cut into steps.  The residual stream, norms, scores and the router are fp32; the matrices and the pool are in the storage dtype.
+#include "stack.h"
+
+#include "kernels/stack.h"
+#include "kernels/stack_gemm.h"
+
+int upload_param_ext(tgx_ctx* c, ebyte* dst, const void* host, int64_t n, int src_dtype);      // abi.hip
+
+namespace {
+
+float half_bits_to_f32(uint16_t h) {
+  const uint32_t s = (h >> 15) & 1, e = (h >> 10) & 0x1f, m = h & 0x3ff;
+  float v = e == 0 ? ldexpf((float)m, -24) : e == 31 ? (m ? NAN : INFINITY) : ldexpf((float)(m | 0x400), (int)e - 25);
+  return s ? -v : v;
+}
+std::vector<float> to_f32(const void* host, int64_t n, int src_dtype) {
+  std::vector<float> out((size_t)n);
+  for (int64_t i = 0; i < n; i++) {
+    if (src_dtype == TGX_F32) out[(size_t)i] = ((const float*)host)[i];
+    else if (src_dtype == TGX_BF16) { const uint32_t u = (uint32_t)((const uint16_t*)host)[i] << 16; memcpy(&out[(size_t)i], &u, 4); }
+    else out[(size_t)i] = half_bits_to_f32(((const uint16_t*)host)[i]);
+  }
+  return out;
+}
+int upload_f32(tgx_ctx* c, float* dst, const void* host, int64_t n, int src_dtype) {
+  const std::vector<float> v = to_f32(host, n, src_dtype);
+  HIP_OK(c, hipMemcpy(dst, v.data(), (size_t)n * 4, hipMemcpyHostToDevice));
+  return TGX_OK;
+}
+size_t esize(int src_dtype) { return src_dtype == TGX_F32 ? 4 : 2; }
+
+struct MetaPtrs { int *tok_id, *tok_pos, *tok_ent, *ent_row, *ent_start, *ent_count, *ent_par, *want, *want_row; size_t n; };
+MetaPtrs meta_layout(int* base, int T, int S, int NW) {
+  MetaPtrs p;
+  p.tok_id = base; p.tok_pos = p.tok_id + T; p.tok_ent = p.tok_pos + T;
+  p.ent_row = p.tok_ent + T; p.ent_start = p.ent_row + S; p.ent_count = p.ent_start + S; p.ent_par = p.ent_count + S;
+  p.want = p.ent_par + S; p.want_row = p.want + NW;
+  p.n = (size_t)3 * T + (size_t)4 * S + (size_t)2 * NW;
+  return p;
+}
+tgx::StepMeta step_meta(const StackModel* sm, const MetaPtrs& p, int T, int S) {
+  tgx::StepMeta m{};
+  m.tok_id = p.tok_id; m.tok_pos = p.tok_pos; m.tok_ent = p.tok_ent; m.ent_row = p.ent_row; m.ent_start = p.ent_start; m.ent_count = p.ent_count; m.ent_par = p.ent_par;
+  m.tbl = sm->tbl_dev; m.tbl_stride = sm->tbl_stride; m.page_shift = sm->page_shift; m.T = T; m.S = S;
+  return m;
+}
+
+// ---- the products --------------------------------------------------------------------------------------------------------------------------
+template <int DT, int EPI, bool DUAL>
+void launch_gemm_t(tgx_ctx* c, const tgx::StackGemmArgs& a, dim3 grid1, dim3 grid2, int wt, bool vec) {
+  auto go = [&](auto WTc, auto VECc) {
+    constexpr int WT = decltype(WTc)::value; constexpr bool VEC = decltype(VECc)::value;
+    const size_t lds = tgx::stack_gemm_lds<DT, DUAL, WT>();
+    hipLaunchKernelGGL((tgx::stack_gemm_kernel<DT, EPI, DUAL, WT, VEC>), WT == 1 ? grid1 : grid2, dim3(256), lds, c->stream, a);
+  };
+  if (wt == 1) { if (vec) go(std::integral_constant<int, 1>{}, std::true_type{}); else go(std::integral_constant<int, 1>{}, std::false_type{}); }
+  else { if (vec) go(std::integral_constant<int, 2>{}, std::true_type{}); else go(std::integral_constant<int, 2>{}, std::false_type{}); }
+}
+// nz: batched products (blockIdx.z); grouped products pass max_tiles_1 = an upper bound of their 64-row tiles (the device-side list says how many are real)
+void launch_gemm(tgx_ctx* c, tgx::StackGemmArgs a, int epi, int nz, int grouped_rows = 0, int groups = 0) {
+  const StackModel* sm = c->stack;
+  if (a.M <= 0 && !a.z_off) return;
+  if (a.N <= 0 || a.K <= 0) return;
+  a.terms = c->act16 ? 1 : 2;
+  const int kq = c->dt == tgx::DT_F32 ? 4 : 8;
+  const bool vec = a.K % kq == 0 && a.ldb % kq == 0 && a.b_zstride % kq == 0 && a.lda % 4 == 0 && a.a_zoff % 4 == 0 && ((uintptr_t)a.A % 16 == 0) && ((uintptr_t)a.B % 16 == 0) &&
+                   (!a.B2 || (uintptr_t)a.B2 % 16 == 0);
+  int wt;
+  dim3 g1, g2;
+  if (a.z_off) {      // grouped: the tile list is built for 64-row tiles
+    wt = 1;
+    g1 = dim3((a.N + 63) / 64, grouped_rows / 64 + groups, 1);
+  } else {
+    g1 = dim3((a.N + 63) / 64, (a.M + 63) / 64, nz);
+    g2 = dim3((a.N + 127) / 128, (a.M + 127) / 128, nz);
+    wt = (size_t)g2.x * g2.y * g2.z >= (size_t)c->num_cus ? 2 : 1;
+    if (sm->gemm_wt) wt = sm->gemm_wt;
+  }
+  const bool dual = epi == tgx::SG_EXPERT_ACT;
+  TGX_DT_SWITCH(c->dt,
+    switch (epi) {
+      case tgx::SG_STORE: launch_gemm_t<DT, tgx::SG_STORE, false>(c, a, g1, g2, wt, vec); break;
+      case tgx::SG_ADD: launch_gemm_t<DT, tgx::SG_ADD, false>(c, a, g1, g2, wt, vec); break;
+      case tgx::SG_GATE: launch_gemm_t<DT, tgx::SG_GATE, false>(c, a, g1, g2, wt, vec); break;
+      case tgx::SG_ROWSCALE: launch_gemm_t<DT, tgx::SG_ROWSCALE, false>(c, a, g1, g2, wt, vec); break;
+      default: if (dual) launch_gemm_t<DT, tgx::SG_EXPERT_ACT, true>(c, a, g1, g2, wt, vec); break;
+    })
+}
+
+template <int DT, bool SPLIT>
+void launch_attn_t(tgx_ctx* c, const tgx::StepMeta& m, const tgx::LatentAttnArgs& a, dim3 grid) {
+  const size_t lds = (size_t)4 * a.rank * 4;
+  const int rpl = (a.rank + 63) / 64;
+  if (rpl <= 1) hipLaunchKernelGGL((tgx::latent_attn_kernel<DT, 1, SPLIT>), grid, dim3(256), lds, c->stream, m, a);
+  else if (rpl <= 2) hipLaunchKernelGGL((tgx::latent_attn_kernel<DT, 2, SPLIT>), grid, dim3(256), lds, c->stream, m, a);
+  else if (rpl <= 4) hipLaunchKernelGGL((tgx::latent_attn_kernel<DT, 4, SPLIT>), grid, dim3(256), lds, c->stream, m, a);
+  else if (rpl <= 8) hipLaunchKernelGGL((tgx::latent_attn_kernel<DT, 8, SPLIT>), grid, dim3(256), lds, c->stream, m, a);
+  else hipLaunchKernelGGL((tgx::latent_attn_kernel<DT, 16, SPLIT>), grid, dim3(256), lds, c->stream, m, a);
+}
+
+int ensure_ws(tgx_ctx* c, int T) {
+  StackModel* sm = c->stack;
+  if (T <= sm->cap_tokens) return TGX_OK;
+  HIP_OK(c, hipStreamSynchronize(c->stream));
+  auto fr = [](auto*& p) { if (p) (void)hipFree(p); p = nullptr; };
+  fr(sm->x); fr(sm->xs); fr(sm->a); fr(sm->proj); fr(sm->ql); fr(sm->lat); fr(sm->o); fr(sm->selw); fr(sm->yh); fr(sm->yd); fr(sm->xn); fr(sm->lg);
+  fr(sm->sel); fr(sm->perm); fr(sm->ptok); fr(sm->tile_e); fr(sm->tile_m0); fr(sm->meta_dev);
+  if (sm->meta_host) { (void)hipHostFree(sm->meta_host); sm->meta_host = nullptr; }
+  const int cap = std::max(T, 64);
+  const size_t W = (size_t)sm->d.width, n = (size_t)cap;
+  int rc;
+  if ((rc = dev_alloc(c, &sm->x, n * W)) || (rc = dev_alloc(c, &sm->xs, (size_t)(sm->d.layers + 1) * n * W)) || (rc = dev_alloc(c, &sm->a, n * W)) ||
+      (rc = dev_alloc(c, &sm->proj, n * (size_t)sm->max_in)) || (rc = dev_alloc(c, &sm->ql, n * (size_t)sm->max_hr)) || (rc = dev_alloc(c, &sm->lat, n * (size_t)sm->max_hr)) ||
+      (rc = dev_alloc(c, &sm->o, n * (size_t)sm->max_hv)) || (rc = dev_alloc(c, &sm->xn, n * W)) || (rc = dev_alloc(c, &sm->lg, n * (size_t)sm->d.vocab))) return rc;
+  if (sm->max_top > 0) {
+    const size_t np = n * (size_t)sm->max_top;
+    if ((rc = dev_alloc(c, &sm->selw, np)) || (rc = dev_alloc(c, &sm->sel, np)) || (rc = dev_alloc(c, &sm->perm, np)) || (rc = dev_alloc(c, &sm->ptok, np)) ||
+        (rc = dev_alloc(c, &sm->yh, np * (size_t)sm->max_ff)) || (rc = dev_alloc(c, &sm->yd, np * W)) ||
+        (rc = dev_alloc(c, &sm->tile_e, np / 64 + (size_t)sm->max_E + 1)) || (rc = dev_alloc(c, &sm->tile_m0, np / 64 + (size_t)sm->max_E + 1))) return rc;
+  }
+  sm->meta_cap = (size_t)5 * n + (size_t)4 * sm->d.max_seqs;
+  if ((rc = dev_alloc(c, &sm->meta_dev, sm->meta_cap))) return rc;
+  HIP_OK(c, hipHostMalloc((void**)&sm->meta_host, sm->meta_cap * 4, hipHostMallocDefault));
+  sm->cap_tokens = cap;
+  return TGX_OK;
+}
+
+int ensure_part(tgx_ctx* c, size_t elems) {
+  StackModel* sm = c->stack;
+  if (elems <= sm->part_elems) return TGX_OK;
+  HIP_OK(c, hipStreamSynchronize(c->stream));
+  if (sm->part) (void)hipFree(sm->part);
+  sm->part = nullptr; sm->part_elems = 0;
+  int rc = dev_alloc(c, &sm->part, elems);
+  if (rc) return rc;
+  sm->part_elems = elems;
+  return TGX_OK;
+}
+
+// the layers of one step; meta is on the device.  max_keys: the longest context any token of the step attends (host knowledge; picks the attention form)
+int run_layers(tgx_ctx* c, const MetaPtrs& mp, int T, int S, int max_keys) {
+  StackModel* sm = c->stack;
+  const tgx::StepMeta m = step_meta(sm, mp, T, S);
+  const int W = sm->d.width, nslots = sm->d.max_seqs, nb = sm->d.canon_taps - 1;
+  const size_t slot_stride = (size_t)sm->cap_tokens * W;
+  TGX_DT_SWITCH(c->dt, hipLaunchKernelGGL(tgx::sinusoid_embed_kernel<DT>, dim3(T), dim3(256), 0, c->stream, m, reinterpret_cast<const tgx::elem_t<DT>*>(c->embed), sm->freq, sm->x, sm->xs, W))
+  for (int li = 0; li < sm->d.layers; li++) {
+    StackLayerW& w = sm->L[(size_t)li];
+    const tgx_layer_desc& ld = w.d;
+    const int H = ld.heads, qd = H * ld.dim, R = ld.kv_rank, vd = H * ld.vdim, nin = qd + R + vd;
+    const size_t st_buf = (size_t)nslots * nb * W;
+    tgx::NormConvArgs nc{};
+    nc.x = sm->x; nc.nw = w.norm1; nc.cw = w.canon1; nc.out = sm->a; nc.state = nb > 0 ? w.conv_state : nullptr; nc.state_buf = st_buf;
+    nc.W = W; nc.groups = sm->d.norm_groups; nc.taps = sm->d.canon_taps; nc.eps = sm->d.norm_eps;
+    hipLaunchKernelGGL(tgx::norm_conv_kernel, dim3(T), dim3(256), 0, c->stream, m, nc);
+    // [q | latent | gate] = a . w_in^T
+    tgx::StackGemmArgs g{};
+    g.A = sm->a; g.lda = W; g.B = w.w_in; g.ldb = W; g.C = sm->proj; g.ldc = nin; g.M = T; g.N = nin; g.K = W; g.scale = 1.f;
+    launch_gemm(c, g, tgx::SG_STORE, 1);
+    tgx::LatentAppendArgs la{};
+    la.src = sm->proj; la.lds = nin; la.col0 = qd; la.nw = w.lat_norm; la.pool = w.pool; la.rank = R; la.eps = sm->d.norm_eps;
+    TGX_DT_SWITCH(c->dt, hipLaunchKernelGGL(tgx::latent_append_kernel<DT>, dim3(T), dim3(64), 0, c->stream, m, la))
+    // queries into latent space, head by head: ql[t][h] = scale * q[t][h] . ukT[h]^T
+    g = tgx::StackGemmArgs{};
+    g.A = sm->proj; g.lda = nin; g.a_zoff = ld.dim; g.B = w.w_ukT; g.ldb = ld.dim; g.b_zstride = (long long)R * ld.dim; g.C = sm->ql; g.ldc = (long long)H * R; g.c_zoff = R;
+    g.M = T; g.N = R; g.K = ld.dim; g.scale = ld.scale;
+    launch_gemm(c, g, tgx::SG_STORE, H);
+    tgx::LatentAttnArgs aa{};
+    aa.q = sm->ql; aa.ldq = (long long)H * R; aa.pool = w.pool; aa.sink = w.sink; aa.out = sm->lat; aa.ldo = (long long)H * R; aa.rank = R; aa.heads = H;
+    int nsplit = 1;
+    if (max_keys >= sm->attn_split_min_keys && (long long)T * H < 2LL * c->num_cus) {
+      nsplit = (int)std::min<long long>(64, (4LL * c->num_cus) / ((long long)T * H));
+      const int per = std::max(256, ((max_keys + nsplit - 1) / nsplit + 63) / 64 * 64);
+      nsplit = (max_keys + per - 1) / per;
+      aa.keys_per = per;
+    }
+    if (nsplit > 1) {
+      int rc = ensure_part(c, (size_t)T * H * nsplit * (size_t)(R + 2));
+      if (rc) return rc;
+      aa.part = sm->part; aa.nsplit = nsplit;
+      TGX_DT_SWITCH(c->dt, (launch_attn_t<DT, true>(c, m, aa, dim3(T, H, nsplit))))
+      hipLaunchKernelGGL(tgx::latent_attn_merge_kernel, dim3(T, H), dim3(256), 0, c->stream, aa);
+    } else {
+      TGX_DT_SWITCH(c->dt, (launch_attn_t<DT, false>(c, m, aa, dim3(T, H))))
+    }
+    // o[t][h] = (lat[t][h] . uv[h]^T) * sigmoid(gate)
+    g = tgx::StackGemmArgs{};
+    g.A = sm->lat; g.lda = (long long)H * R; g.a_zoff = R; g.B = w.w_uv; g.ldb = R; g.b_zstride = (long long)ld.vdim * R; g.C = sm->o; g.ldc = vd; g.c_zoff = ld.vdim;
+    g.M = T; g.N = ld.vdim; g.K = R; g.G = sm->proj; g.ldg = nin; g.g_col0 = qd + R;
+    launch_gemm(c, g, tgx::SG_GATE, H);
+    // x += o . w_o^T
+    g = tgx::StackGemmArgs{};
+    g.A = sm->o; g.lda = vd; g.B = w.w_o; g.ldb = vd; g.C = sm->x; g.ldc = W; g.M = T; g.N = W; g.K = vd;
+    launch_gemm(c, g, tgx::SG_ADD, 1);
+    int top = 0;
+    if (ld.mlp == TGX_MLP_MOE) {
+      top = ld.top;
+      nc.nw = w.norm2; nc.cw = w.canon2; nc.state = nb > 0 ? w.conv_state + 2 * st_buf : nullptr;
+      hipLaunchKernelGGL(tgx::norm_conv_kernel, dim3(T), dim3(256), 0, c->stream, m, nc);
+      tgx::RouterArgs ra{};
+      ra.h = sm->a; ra.wr = w.w_router; ra.br = w.b_router; ra.sel = sm->sel; ra.selw = sm->selw; ra.W = W; ra.E = ld.experts; ra.top = top;
+      hipLaunchKernelGGL(tgx::router_topk_kernel, dim3(T), dim3(256), 0, c->stream, ra);
+      const int np = T * top;
+      tgx::MoePlanArgs pa{};
+      pa.sel = sm->sel; pa.n_pairs = np; pa.E = ld.experts; pa.top = top; pa.tile_m = 64;
+      pa.off = sm->moe_off; pa.perm = sm->perm; pa.tok = sm->ptok; pa.tile_e = sm->tile_e; pa.tile_m0 = sm->tile_m0; pa.n_tiles = sm->n_tiles;
+      hipLaunchKernelGGL(tgx::moe_plan_kernel, dim3(1), dim3(1024), 0, c->stream, pa);
+      // yh[n] = act(gate_e . a[tok(n)], up_e . a[tok(n)]) over the pairs grouped by expert
+      g = tgx::StackGemmArgs{};
+      g.A = sm->a; g.lda = W; g.a_rows = sm->ptok; g.B = w.w_gate; g.B2 = w.w_up; g.ldb = W; g.b_zstride = (long long)ld.ff * W; g.C = sm->yh; g.ldc = ld.ff;
+      g.z_off = sm->moe_off; g.tile_z = sm->tile_e; g.tile_m0 = sm->tile_m0; g.n_tiles = sm->n_tiles; g.M = np; g.N = ld.ff; g.K = W; g.limit = ld.limit;
+      launch_gemm(c, g, tgx::SG_EXPERT_ACT, 1, np, ld.experts);
+      // yd[pair] = router weight * (down_e . yh[n])
+      g = tgx::StackGemmArgs{};
+      g.A = sm->yh; g.lda = ld.ff; g.B = w.w_down; g.ldb = ld.ff; g.b_zstride = (long long)W * ld.ff; g.C = sm->yd; g.ldc = W; g.c_rows = sm->perm;
+      g.z_off = sm->moe_off; g.tile_z = sm->tile_e; g.tile_m0 = sm->tile_m0; g.n_tiles = sm->n_tiles; g.M = np; g.N = W; g.K = ld.ff; g.rw = sm->selw;
+      launch_gemm(c, g, tgx::SG_ROWSCALE, 1, np, ld.experts);
+    }
+    tgx::CombineDepthArgs cd{};
+    cd.x = sm->x; cd.y = sm->yd; cd.xs = sm->xs; cd.slot_stride = slot_stride; cd.dw = w.dwa; cd.W = W; cd.top = top; cd.n_res = li + 2;
+    hipLaunchKernelGGL(tgx::combine_depth_kernel, dim3(T), dim3(256), 0, c->stream, cd);
+  }
+  return TGX_OK;
+}
+
+// logits of the rows listed in want_dev (indices into the step's tokens): C[crow(i)] = embed . norm(x[want[i]]) * logit_scale
+void run_logits(tgx_ctx* c, const int* want_dev, int nw, float* C, const int* c_rows) {
+  StackModel* sm = c->stack;
+  const int W = sm->d.width, V = sm->d.vocab;
+  hipLaunchKernelGGL(tgx::final_norm_rows_kernel, dim3(nw), dim3(256), 0, c->stream, sm->x, want_dev, sm->final_norm, sm->xn, W, sm->d.norm_groups, sm->d.norm_eps);
+  tgx::StackGemmArgs g{};
+  g.A = sm->xn; g.lda = W; g.B = c->embed; g.ldb = W; g.C = C; g.ldc = V; g.c_rows = c_rows; g.M = nw; g.N = V; g.K = W; g.scale = sm->d.logit_scale;
+  launch_gemm(c, g, tgx::SG_STORE, 1);
+}
+
+// pages for `tokens` tokens of a slot; the caller has checked that enough are free
+void assign_pages(StackModel* sm, int row, long long tokens) {
+  const int need = (int)((tokens + sm->page - 1) / sm->page);
+  int& have = sm->row_pages[(size_t)row];
+  for (; have < need; have++) {
+    sm->tbl_host[(size_t)row * sm->tbl_stride + have] = sm->free_pages.back();
+    sm->free_pages.pop_back();
+    sm->row_dirty[(size_t)row] = 1;
+  }
+}
+int push_tables(tgx_ctx* c) {
+  StackModel* sm = c->stack;
+  for (int r = 0; r < sm->d.max_seqs; r++)
+    if (sm->row_dirty[(size_t)r]) {
+      const size_t o = (size_t)r * sm->tbl_stride;
+      HIP_OK(c, hipMemcpyAsync(sm->tbl_dev + o, sm->tbl_host + o, (size_t)std::max(1, sm->row_pages[(size_t)r]) * 4, hipMemcpyHostToDevice, c->stream));
+      sm->row_dirty[(size_t)r] = 0;
+    }
+  return TGX_OK;
+}
+int push_meta(tgx_ctx* c, size_t n) {
+  StackModel* sm = c->stack;
+  HIP_OK(c, hipMemcpyAsync(sm->meta_dev, sm->meta_host, n * 4, hipMemcpyHostToDevice, c->stream));
+  HIP_OK(c, hipEventRecord(sm->meta_ev, c->stream));
+  sm->meta_pending = true;
+  return TGX_OK;
+}
+int meta_host_free(tgx_ctx* c) {      // the pinned staging block may be rewritten once the last copy out of it has run
+  StackModel* sm = c->stack;
+  if (sm->meta_pending) { HIP_OK(c, hipEventSynchronize(sm->meta_ev)); sm->meta_pending = false; }
+  return TGX_OK;
+}
+
+void refresh_rows(tgx_ctx* c) {
+  int64_t m = 0; int live = 0; bool all = true;
+  for (int b = 0; b < c->batch; b++) {
+    if (c->row_idle[(size_t)b]) continue;
+    live++; m = std::max(m, c->row_past[(size_t)b]); all = all && c->row_tok[(size_t)b];
+  }
+  c->past = m; c->have_token = live > 0 && all;
+}
+
+}  // namespace
+
+// ================================================================================================================================================
+int stack_create(const tgx_stack_desc* desc, const tgx_layer_desc* layers, int device_ordinal, tgx_ctx** out_ctx) {
+  if (!desc || !layers || !out_ctx) return set_err(nullptr, TGX_ERR_INVALID, "null argument");
+  *out_ctx = nullptr;
+  const tgx_stack_desc& d = *desc;
+  if (d.family != TGX_FAMILY_ZAKUSUN) return set_err(nullptr, TGX_ERR_UNSUPPORTED, "family %d is not a layered model", d.family);
+  if (d.width <= 0 || d.layers <= 0 || d.vocab <= 0 || d.max_seqs <= 0 || d.max_ctx <= 0) return set_err(nullptr, TGX_ERR_INVALID, "non-positive model dimension");
+  if (d.compute_dtype != TGX_BF16 && d.compute_dtype != TGX_F16 && d.compute_dtype != TGX_F32) return set_err(nullptr, TGX_ERR_INVALID, "unknown compute dtype %d", d.compute_dtype);
+  if (d.norm_groups < 1 || d.norm_groups > tgx::NORM_MAX_GROUPS || d.width % d.norm_groups) return set_err(nullptr, TGX_ERR_UNSUPPORTED, "norm groups %d: 1..%d, dividing the width", d.norm_groups, tgx::NORM_MAX_GROUPS);
+  if (d.canon_taps < 1 || d.canon_taps > tgx::CONV_MAX_TAPS) return set_err(nullptr, TGX_ERR_UNSUPPORTED, "convolution taps %d: 1..%d", d.canon_taps, tgx::CONV_MAX_TAPS);
+  int page = d.page_tokens > 0 ? d.page_tokens : 64;
+  if (page & (page - 1)) return set_err(nullptr, TGX_ERR_INVALID, "page_tokens %d is not a power of two", page);
+  for (int i = 0; i < d.layers; i++) {
+    const tgx_layer_desc& l = layers[i];
+    if (l.mixer != TGX_MIXER_LATENT_ATTENTION) return set_err(nullptr, TGX_ERR_UNSUPPORTED, "layer %d: mixer %d is not implemented (latent_attention is)", i, l.mixer);
+    if (l.heads <= 0 || l.dim <= 0 || l.vdim <= 0 || l.kv_rank <= 0) return set_err(nullptr, TGX_ERR_INVALID, "layer %d: non-positive mixer size", i);
+    if (l.kv_rank > 64 * tgx::LAT_MAX_RPL) return set_err(nullptr, TGX_ERR_UNSUPPORTED, "layer %d: kv_rank %d > %d", i, l.kv_rank, 64 * tgx::LAT_MAX_RPL);
+    if (l.mlp != TGX_MLP_NONE && l.mlp != TGX_MLP_MOE) return set_err(nullptr, TGX_ERR_UNSUPPORTED, "layer %d: feed-forward kind %d is not implemented", i, l.mlp);
+    if (l.mlp == TGX_MLP_MOE && (l.experts <= 0 || l.experts > tgx::ROUTER_MAX_E || l.top <= 0 || l.top > l.experts || l.top > tgx::ROUTER_MAX_TOP || l.ff <= 0))
+      return set_err(nullptr, TGX_ERR_UNSUPPORTED, "layer %d: experts %d (<= %d), top %d (<= %d), ff %d", i, l.experts, tgx::ROUTER_MAX_E, l.top, tgx::ROUTER_MAX_TOP, l.ff);
+  }
+  int ndev = 0;
+  if (hipGetDeviceCount(&ndev) != hipSuccess || ndev <= 0) return set_err(nullptr, TGX_ERR_DEVICE, "no HIP device visible (--device mi355x needs a GPU; there is no CPU fallback)");
+  if (device_ordinal < 0 || device_ordinal >= ndev) return set_err(nullptr, TGX_ERR_INVALID, "device ordinal %d out of range [0,%d)", device_ordinal, ndev);
+
+  tgx_ctx* c = new (std::nothrow) tgx_ctx();
+  StackModel* sm = new (std::nothrow) StackModel();
+  if (!c || !sm) { delete c; delete sm; return set_err(nullptr, TGX_ERR_NOMEM, "host allocation failed"); }
+  *out_ctx = c;
+  c->stack = sm;
+  sm->d = d;
+  sm->page = page; sm->page_shift = 0;
+  while ((1 << sm->page_shift) < page) sm->page_shift++;
+  // what the shared sampler / token rings read from the flat description
+  c->d.family = d.family; c->d.hidden = d.width; c->d.layers = d.layers; c->d.vocab = d.vocab; c->d.max_ctx = d.max_ctx; c->d.max_batch = d.max_seqs;
+  c->d.compute_dtype = d.compute_dtype; c->d.tied = 1; c->d.norm_eps = d.norm_eps;
+  c->device = device_ordinal;
+  c->dt = d.compute_dtype == TGX_BF16 ? tgx::DT_BF16 : (d.compute_dtype == TGX_F16 ? tgx::DT_F16 : tgx::DT_F32);
+  c->esz = d.compute_dtype == TGX_F32 ? 4 : 2;
+  HIP_OK(c, hipSetDevice(device_ordinal));
+  hipDeviceProp_t prop;
+  HIP_OK(c, hipGetDeviceProperties(&prop, device_ordinal));
+  c->num_cus = prop.multiProcessorCount > 0 ? prop.multiProcessorCount : 256;
+  HIP_OK(c, hipStreamCreateWithFlags(&c->stream, hipStreamNonBlocking));
+
+  const size_t W = (size_t)d.width, es = c->esz;
+  int rc;
+  if ((rc = dev_alloc(c, &c->embed, (size_t)d.vocab * W * es)) || (rc = dev_alloc(c, &sm->final_norm, W))) return rc;
+  sm->missing.insert("embed"); sm->missing.insert("final.norm");
+  sm->L.resize((size_t)d.layers);
+  for (int i = 0; i < d.layers; i++) {
+    StackLayerW& w = sm->L[(size_t)i];
+    w.d = layers[i];
+    const tgx_layer_desc& l = w.d;
+    const std::string p = "l" + std::to_string(i) + ".";
+    const size_t H = (size_t)l.heads, qd = H * l.dim, R = (size_t)l.kv_rank, vd = H * l.vdim;
+    if ((rc = dev_alloc(c, &w.norm1, W)) || (rc = dev_alloc(c, &w.dwa, (size_t)i + 2)) || (rc = dev_alloc(c, &w.w_in, (qd + R + vd) * W * es)) ||
+        (rc = dev_alloc(c, &w.w_ukT, qd * R * es)) || (rc = dev_alloc(c, &w.w_uv, vd * R * es)) || (rc = dev_alloc(c, &w.w_o, W * vd * es)) ||
+        (rc = dev_alloc(c, &w.lat_norm, R)) || (rc = dev_alloc(c, &w.sink, H))) return rc;
+    for (const char* n : {"norm1", "dwa", "mix.q", "mix.dkv", "mix.dkv.norm", "mix.uk", "mix.uv", "mix.sink", "mix.g", "mix.o"}) sm->missing.insert(p + n);
+    if (d.canon_taps > 1) { if ((rc = dev_alloc(c, &w.canon1, W * d.canon_taps))) return rc; sm->missing.insert(p + "canon1"); }
+    if (l.mlp == TGX_MLP_MOE) {
+      const size_t E = (size_t)l.experts, F = (size_t)l.ff;
+      if ((rc = dev_alloc(c, &w.norm2, W)) || (rc = dev_alloc(c, &w.w_gate, E * F * W * es)) || (rc = dev_alloc(c, &w.w_up, E * F * W * es)) ||
+          (rc = dev_alloc(c, &w.w_down, E * W * F * es)) || (rc = dev_alloc(c, &w.w_router, E * W)) || (rc = dev_alloc(c, &w.b_router, E))) return rc;
+      for (const char* n : {"norm2", "mlp.router", "mlp.router.b"}) sm->missing.insert(p + n);
+      if (d.canon_taps > 1) { if ((rc = dev_alloc(c, &w.canon2, W * d.canon_taps))) return rc; sm->missing.insert(p + "canon2"); }
+      for (int e = 0; e < l.experts; e++)
+        for (const char* n : {".gate", ".up", ".down"}) sm->missing.insert(p + "mlp.e" + std::to_string(e) + n);
+      sm->max_top = std::max(sm->max_top, l.top); sm->max_ff = std::max(sm->max_ff, l.ff); sm->max_E = std::max(sm->max_E, l.experts);
+    }
+    sm->max_in = std::max(sm->max_in, (int)(qd + R + vd)); sm->max_hr = std::max(sm->max_hr, (int)(H * R)); sm->max_hv = std::max(sm->max_hv, (int)vd);
+    sm->max_rank = std::max(sm->max_rank, l.kv_rank);
+  }
+  return TGX_OK;
+}
+
+int stack_upload(tgx_ctx* c, const char* name, const void* host, const int64_t* shape, int nd, int src_dtype) {
+  StackModel* sm = c->stack;
+  const tgx_stack_desc& d = sm->d;
+  const int64_t W = d.width;
+  auto bad_shape = [&]() { return set_err(c, TGX_ERR_SHAPE, "shape not equal for tensor: %s", name); };
+  auto is = [&](int64_t a, int64_t b) { return b < 0 ? (nd == 1 && shape[0] == a) : (nd == 2 && shape[0] == a && shape[1] == b); };
+  const bool probe = nd < 0;      // name lookup only (include/tgx.h): every tensor this model knows is a parameter it needs
+  auto done = [&](int rc) { if (!rc) sm->missing.erase(name); return rc; };
+  if (src_dtype != TGX_BF16 && src_dtype != TGX_F32 && src_dtype != TGX_F16) return set_err(c, TGX_ERR_INVALID, "unknown source dtype %d", src_dtype);
+  if (!strcmp(name, "embed")) { if (probe) return TGX_ERR_SHAPE; if (!is(d.vocab, W)) return bad_shape(); return done(upload_param_ext(c, c->embed, host, d.vocab * W, src_dtype)); }
+  if (!strcmp(name, "final.norm")) { if (probe) return TGX_ERR_SHAPE; if (!is(W, -1)) return bad_shape(); return done(upload_f32(c, sm->final_norm, host, W, src_dtype)); }
+  int li = -1;
+  char rest[128] = {0};
+  if (sscanf(name, "l%d.%127s", &li, rest) != 2 || li < 0 || li >= d.layers) return set_err(c, TGX_ERR_NAME, "Unexpected key: %s", name);
+  StackLayerW& w = sm->L[(size_t)li];
+  const tgx_layer_desc& l = w.d;
+  const int64_t H = l.heads, qd = H * l.dim, R = l.kv_rank, vd = H * l.vdim, E = l.experts, F = l.ff;
+  struct F32Slot { const char* n; float* dst; int64_t a, b; };
+  const F32Slot fs[] = {{"norm1", w.norm1, W, -1}, {"norm2", w.norm2, W, -1}, {"canon1", w.canon1, W, d.canon_taps}, {"canon2", w.canon2, W, d.canon_taps},
+                        {"dwa", w.dwa, li + 2, -1}, {"mix.dkv.norm", w.lat_norm, R, -1}, {"mix.sink", w.sink, H, -1},
+                        {"mlp.router", w.w_router, E, W}, {"mlp.router.b", w.b_router, E, -1}};
+  for (const F32Slot& s : fs)
+    if (!strcmp(rest, s.n)) {
+      if (!s.dst) break;
+      if (probe) return TGX_ERR_SHAPE;
+      if (!is(s.a, s.b)) return bad_shape();
+      return done(upload_f32(c, s.dst, host, s.b < 0 ? s.a : s.a * s.b, src_dtype));
+    }
+  struct MatSlot { const char* n; ebyte* dst; int64_t row0, rows, cols; };
+  const MatSlot ms[] = {{"mix.q", w.w_in, 0, qd, W}, {"mix.dkv", w.w_in, qd, R, W}, {"mix.g", w.w_in, qd + R, vd, W}, {"mix.uv", w.w_uv, 0, vd, R}, {"mix.o", w.w_o, 0, W, vd}};
+  for (const MatSlot& s : ms)
+    if (!strcmp(rest, s.n)) {
+      if (probe) return TGX_ERR_SHAPE;
+      if (!is(s.rows, s.cols)) return bad_shape();
+      return done(upload_param_ext(c, s.dst + (size_t)(s.row0 * s.cols) * c->esz, host, s.rows * s.cols, src_dtype));
+    }
+  if (!strcmp(rest, "mix.uk")) {      // [heads * dim][rank] -> per head [rank][dim]
+    if (probe) return TGX_ERR_SHAPE;
+    if (!is(qd, R)) return bad_shape();
+    const size_t es = esize(src_dtype);
+    std::vector<unsigned char> t((size_t)(qd * R) * es);
+    const unsigned char* src = (const unsigned char*)host;
+    for (int64_t h = 0; h < H; h++)
+      for (int64_t dd = 0; dd < l.dim; dd++)
+        for (int64_t r = 0; r < R; r++) memcpy(&t[(size_t)((h * R + r) * l.dim + dd) * es], src + (size_t)((h * l.dim + dd) * R + r) * es, es);
+    return done(upload_param_ext(c, w.w_ukT, t.data(), qd * R, src_dtype));
+  }
+  int e = -1;
+  char leaf[32] = {0};
+  if (l.mlp == TGX_MLP_MOE && sscanf(rest, "mlp.e%d.%31s", &e, leaf) == 2 && e >= 0 && e < E) {
+    if (probe) return TGX_ERR_SHAPE;
+    if (!strcmp(leaf, "gate") || !strcmp(leaf, "up")) {
+      if (!is(F, W)) return bad_shape();
+      return done(upload_param_ext(c, (leaf[0] == 'g' ? w.w_gate : w.w_up) + (size_t)(e * F * W) * c->esz, host, F * W, src_dtype));
+    }
+    if (!strcmp(leaf, "down")) {
+      if (!is(W, F)) return bad_shape();
+      return done(upload_param_ext(c, w.w_down + (size_t)(e * W * F) * c->esz, host, W * F, src_dtype));
+    }
+  }
+  return set_err(c, TGX_ERR_NAME, "Unexpected key: %s", name);
+}
+
+int stack_finalize(tgx_ctx* c) {
+  StackModel* sm = c->stack;
+  const tgx_stack_desc& d = sm->d;
+  if (!sm->missing.empty()) return set_err(c, TGX_ERR_STATE, "Missing key: %s", sm->missing.begin()->c_str());
+  if (c->finalized) return TGX_OK;
+  HIP_OK(c, hipSetDevice(c->device));
+  const size_t W = (size_t)d.width, B = (size_t)d.max_seqs, V = (size_t)d.vocab;
+  int rc;
+  // angles of the position vector: pos * base^(-2i / width), the factor rounded to fp32 once
+  std::vector<float> fq(W / 2 + 1);
+  for (size_t i = 0; i < fq.size(); i++) fq[i] = (float)pow(10000.0, -2.0 * (double)i / (double)W);
+  if ((rc = dev_alloc(c, &sm->freq, fq.size()))) return rc;
+  HIP_OK(c, hipMemcpy(sm->freq, fq.data(), fq.size() * 4, hipMemcpyHostToDevice));
+  // the latent pool and its page tables
+  const long long budget = d.budget_tokens > 0 ? d.budget_tokens : (long long)d.max_seqs * d.max_ctx;
+  sm->n_pages = (int)((budget + sm->page - 1) / sm->page);
+  sm->tbl_stride = (d.max_ctx + sm->page - 1) / sm->page;
+  if ((rc = dev_alloc(c, &sm->tbl_dev, B * (size_t)sm->tbl_stride))) return rc;
+  HIP_OK(c, hipMemset(sm->tbl_dev, 0, B * (size_t)sm->tbl_stride * 4));
+  HIP_OK(c, hipHostMalloc((void**)&sm->tbl_host, B * (size_t)sm->tbl_stride * 4, hipHostMallocDefault));
+  memset(sm->tbl_host, 0, B * (size_t)sm->tbl_stride * 4);
+  sm->row_pages.assign(B, 0); sm->row_par.assign(B, 0); sm->row_dirty.assign(B, 0);
+  for (int p = sm->n_pages - 1; p >= 0; p--) sm->free_pages.push_back(p);
+  const size_t nb = (size_t)d.canon_taps - 1;
+  for (auto& w : sm->L) {
+    const size_t pe = (size_t)sm->n_pages * sm->page * (size_t)w.d.kv_rank * c->esz;
+    if ((rc = dev_alloc(c, &w.pool, pe))) return rc;
+    HIP_OK(c, hipMemset(w.pool, 0, pe));
+    if (nb > 0) {
+      const size_t se = 4 * B * nb * W;
+      if ((rc = dev_alloc(c, &w.conv_state, se))) return rc;
+      HIP_OK(c, hipMemset(w.conv_state, 0, se * 4));
+    }
+  }
+  if ((rc = dev_alloc(c, &sm->moe_off, (size_t)sm->max_E + 2)) || (rc = dev_alloc(c, &sm->n_tiles, 1))) return rc;
+  HIP_OK(c, hipEventCreateWithFlags(&sm->meta_ev, hipEventDisableTiming));
+  // the rows of the shared sampler (logits, argmax partials, current token) and the token rings
+  c->lm_grid = gemv_grid(c, (int)(V + 1) / 2, 1, c->tune[TGX_KERNEL_LMHEAD].bpc);
+  c->rows.resize(B);
+  if ((rc = dev_alloc(c, &c->slab_x, B * W)) || (rc = dev_alloc(c, &c->slab_logits, B * V)) || (rc = dev_alloc(c, &c->slab_probs, B * V)) ||
+      (rc = dev_alloc(c, &c->slab_part_val, B * c->lm_grid)) || (rc = dev_alloc(c, &c->slab_part_idx, B * c->lm_grid)) || (rc = dev_alloc(c, &c->slab_tok, B)) ||
+      (rc = dev_alloc(c, &c->slab_pos, B))) return rc;
+  HIP_OK(c, hipMemset(c->slab_tok, 0, B * 4));
+  HIP_OK(c, hipMemset(c->slab_pos, 0, B * 4));
+  HIP_OK(c, hipMemset(c->slab_part_val, 0, B * c->lm_grid * 4));      // a slot that never held logits still rides through the sampler: it picks token 0
+  HIP_OK(c, hipMemset(c->slab_part_idx, 0, B * c->lm_grid * 4));
+  HIP_OK(c, hipMemset(c->slab_logits, 0, B * V * 4));
+  for (size_t b = 0; b < B; b++) {
+    RowState& r = c->rows[b];
+    r.x = c->slab_x + b * W; r.logits = c->slab_logits + b * V; r.probs = c->slab_probs + b * V;
+    r.part_val = c->slab_part_val + b * c->lm_grid; r.part_idx = c->slab_part_idx + b * c->lm_grid; r.tok = c->slab_tok + b; r.pos = c->slab_pos + b;
+  }
+  c->log_cap = d.max_ctx > 1024 ? d.max_ctx : 1024;
+  if ((rc = dev_alloc(c, &c->step, 1)) || (rc = dev_alloc(c, &c->step_done, 1)) || (rc = dev_alloc(c, &c->seed_dev, 1)) || (rc = sampler_alloc(c)) ||
+      (rc = dev_alloc(c, &c->tok_log, (size_t)c->log_cap * B))) return rc;
+  HIP_OK(c, hipMemset(c->step, 0, 4));
+  HIP_OK(c, hipMemset(c->step_done, 0, 4));
+  HIP_OK(c, hipHostMalloc((void**)&c->host_ring, (size_t)HOST_RING * B * 4, hipHostMallocMapped));
+  HIP_OK(c, hipHostGetDevicePointer((void**)&c->host_ring_dev, c->host_ring, 0));
+  for (int i = 0; i < MAX_TICKET_EVENTS; i++) HIP_OK(c, hipEventCreateWithFlags(&c->ticket_ev[i], hipEventDisableTiming));
+  c->past = 0;
+  c->row_past.assign(B, 0); c->row_tok.assign(B, 0); c->row_idle.assign(B, 0);
+  c->row_probs_cfg.resize(B); c->row_probs_ok.assign(B, 0);
+  c->finalized = true;
+  return TGX_OK;
+}
+
+void stack_destroy(tgx_ctx* c) {
+  StackModel* sm = c->stack;
+  if (!sm) return;
+  auto fr = [](void* p) { if (p) (void)hipFree(p); };
+  for (auto& w : sm->L) {
+    fr(w.norm1); fr(w.norm2); fr(w.canon1); fr(w.canon2); fr(w.dwa); fr(w.w_in); fr(w.w_ukT); fr(w.w_uv); fr(w.w_o); fr(w.lat_norm); fr(w.sink);
+    fr(w.w_gate); fr(w.w_up); fr(w.w_down); fr(w.w_router); fr(w.b_router); fr(w.pool); fr(w.conv_state);
+  }
+  fr(sm->final_norm); fr(sm->freq); fr(sm->tbl_dev); fr(sm->meta_dev); fr(sm->x); fr(sm->xs); fr(sm->a); fr(sm->proj); fr(sm->ql); fr(sm->lat); fr(sm->o); fr(sm->selw);
+  fr(sm->yh); fr(sm->yd); fr(sm->xn); fr(sm->lg); fr(sm->part); fr(sm->sel); fr(sm->moe_off); fr(sm->perm); fr(sm->ptok); fr(sm->tile_e); fr(sm->tile_m0); fr(sm->n_tiles);
+  if (sm->tbl_host) (void)hipHostFree(sm->tbl_host);
+  if (sm->meta_host) (void)hipHostFree(sm->meta_host);
+  if (sm->meta_ev) (void)hipEventDestroy(sm->meta_ev);
+  delete sm;
+  c->stack = nullptr;
+}
+
+int stack_free_tokens(const tgx_ctx* c) { return (int)std::min<long long>(INT32_MAX, (long long)c->stack->free_pages.size() * c->stack->page); }
+
+int stack_reset_row(tgx_ctx* c, int row) {
+  StackModel* sm = c->stack;
+  HIP_OK(c, hipStreamSynchronize(c->stream));      // nothing in flight reads the slot's pages or its table any more
+  int& have = sm->row_pages[(size_t)row];
+  for (int b = 0; b < have; b++) sm->free_pages.push_back(sm->tbl_host[(size_t)row * sm->tbl_stride + b]);
+  have = 0;
+  c->row_past[(size_t)row] = 0; c->row_tok[(size_t)row] = 0;
+  c->row_idle[(size_t)row] = row < c->batch;
+  while (c->batch > 0 && c->row_idle[(size_t)c->batch - 1]) { c->row_idle[(size_t)c->batch - 1] = 0; c->batch--; }      // trailing free slots leave the batch
+  refresh_rows(c);
+  return TGX_OK;
+}
+
+int stack_step(tgx_ctx* c, int S, const int32_t* rows, const int32_t* counts, const int64_t* ids, int n_want, const int32_t* want, float* out_logits) {
+  StackModel* sm = c->stack;
+  const tgx_stack_desc& d = sm->d;
+  if (S < 1 || S > d.max_seqs || !rows || !counts || !ids || n_want < 0 || (n_want > 0 && (!want || !out_logits))) return set_err(c, TGX_ERR_INVALID, "step: bad argument");
+  long long T = 0, need_pages = 0;
+  int max_keys = 0;
+  std::vector<char> seen((size_t)d.max_seqs, 0);
+  for (int e = 0; e < S; e++) {
+    const int r = rows[e];
+    if (r < 0 || r >= d.max_seqs || seen[(size_t)r]) return set_err(c, TGX_ERR_INVALID, "step: slot %d out of range [0,%d) or listed twice", r, d.max_seqs);
+    seen[(size_t)r] = 1;
+    if (counts[e] < 1) return set_err(c, TGX_ERR_INVALID, "step: entry %d brings no token", e);
+    const long long after = c->row_past[(size_t)r] + counts[e];
+    if (after > d.max_ctx) return set_err(c, TGX_ERR_CONTEXT, "context size exceeded: slot %d would hold %lld tokens (contextSize %d)", r, after, d.max_ctx);
+    need_pages += std::max<long long>(0, (after + sm->page - 1) / sm->page - sm->row_pages[(size_t)r]);
+    max_keys = std::max<int>(max_keys, (int)after);
+    T += counts[e];
+  }
+  if (T > (1 << 24)) return set_err(c, TGX_ERR_INVALID, "step: %lld tokens", T);
+  for (long long i = 0; i < T; i++) if (ids[i] < 0 || ids[i] >= d.vocab) return set_err(c, TGX_ERR_INVALID, "token id out of range");
+  for (int i = 0; i < n_want; i++) if (want[i] < 0 || want[i] >= T) return set_err(c, TGX_ERR_INVALID, "step: wanted index %d outside the step's %lld tokens", want[i], T);
+  if (need_pages > (long long)sm->free_pages.size())
+    return set_err(c, TGX_ERR_CONTEXT, "latent pool exhausted: the step needs %lld more pages of %d tokens, %zu free of %d", need_pages, sm->page, sm->free_pages.size(), sm->n_pages);
+  HIP_OK(c, hipSetDevice(c->device));
+  int rc;
+  if ((rc = ensure_ws(c, (int)std::max<long long>(T, n_want)))) return rc;
+  if ((rc = meta_host_free(c))) return rc;
+  const MetaPtrs hp = meta_layout(sm->meta_host, (int)T, S, n_want), dp = meta_layout(sm->meta_dev, (int)T, S, n_want);
+  std::vector<int> last_want((size_t)S, -1);
+  int t = 0;
+  for (int e = 0; e < S; e++) {
+    const int r = rows[e];
+    assign_pages(sm, r, c->row_past[(size_t)r] + counts[e]);
+    hp.ent_row[e] = r; hp.ent_start[e] = t; hp.ent_count[e] = counts[e]; hp.ent_par[e] = sm->row_par[(size_t)r];
+    for (int i = 0; i < counts[e]; i++, t++) { hp.tok_id[t] = (int)ids[t]; hp.tok_pos[t] = (int)c->row_past[(size_t)r] + i; hp.tok_ent[t] = e; }
+  }
+  for (int i = 0; i < n_want; i++) {
+    hp.want[i] = want[i]; hp.want_row[i] = 0;
+    for (int e = 0; e < S; e++) if (want[i] == hp.ent_start[e] + counts[e] - 1) last_want[(size_t)e] = i;
+  }
+  if ((rc = push_tables(c)) || (rc = push_meta(c, hp.n))) return rc;
+  if ((rc = run_layers(c, dp, (int)T, S, max_keys))) return rc;
+  if (n_want > 0) {
+    run_logits(c, dp.want, n_want, sm->lg, nullptr);
+    HIP_OK(c, hipMemcpyAsync(out_logits, sm->lg, (size_t)n_want * d.vocab * 4, hipMemcpyDeviceToHost, c->stream));
+  }
+  for (int e = 0; e < S; e++) {
+    const int r = rows[e];
+    if (last_want[(size_t)e] >= 0) {      // the slot's current logits: what tgx_sample_row / tgx_read_logits see
+      HIP_OK(c, hipMemcpyAsync(c->rows[(size_t)r].logits, sm->lg + (size_t)last_want[(size_t)e] * d.vocab, (size_t)d.vocab * 4, hipMemcpyDeviceToDevice, c->stream));
+      launch_argmax_partials(c, c->rows[(size_t)r].logits, d.vocab, c->rows[(size_t)r].part_val, c->rows[(size_t)r].part_idx);
+      c->have_logits = true;
+    }
+  }
+  HIP_OK(c, hipGetLastError());
+  HIP_OK(c, hipStreamSynchronize(c->stream));
+  for (int e = 0; e < S; e++) {
+    const int r = rows[e];
+    c->row_past[(size_t)r] += counts[e];
+    sm->row_par[(size_t)r] ^= 1;
+    c->row_tok[(size_t)r] = 0; c->row_idle[(size_t)r] = 0;
+    c->batch = std::max(c->batch, r + 1);
+    if ((size_t)r < c->row_probs_ok.size()) c->row_probs_ok[(size_t)r] = 0;
+  }
+  for (int b = 0; b < c->batch; b++) if (!seen[(size_t)b] && c->row_past[(size_t)b] == 0 && !c->row_idle[(size_t)b]) c->row_idle[(size_t)b] = 1;      // slots below a newly admitted one that hold nothing
+  refresh_rows(c);
+  return TGX_OK;
+}
+
+// n decode steps of every live slot: its device-resident current token in, logits into its row, the shared sampler picks the next token
+int stack_decode(tgx_ctx* c, const tgx_sampler_cfg& cfg, uint64_t seed, int n) {
+  StackModel* sm = c->stack;
+  const tgx_stack_desc& d = sm->d;
+  if (n <= 0) return TGX_OK;
+  std::vector<int> live;
+  long long need_pages = 0;
+  int max_keys = 0;
+  for (int b = 0; b < c->batch; b++) {
+    if (c->row_idle[(size_t)b]) continue;
+    live.push_back(b);
+    const long long after = c->row_past[(size_t)b] + n;
+    need_pages += std::max<long long>(0, (after + sm->page - 1) / sm->page - sm->row_pages[(size_t)b]);
+    max_keys = std::max<int>(max_keys, (int)c->row_past[(size_t)b]);
+  }
+  if (live.empty()) return set_err(c, TGX_ERR_STATE, "decode: every slot is retired");
+  if (need_pages > (long long)sm->free_pages.size())
+    return set_err(c, TGX_ERR_CONTEXT, "latent pool exhausted: %d decode steps need %lld more pages of %d tokens, %zu free", n, need_pages, sm->page, sm->free_pages.size());
+  if (!is_greedy(&cfg) && (!c->seed_valid || c->seed_on_dev != (unsigned long long)seed)) {
+    HIP_OK(c, hipStreamSynchronize(c->stream));
+    const unsigned long long s = seed;
+    HIP_OK(c, hipMemcpy(c->seed_dev, &s, 8, hipMemcpyHostToDevice));
+    c->seed_on_dev = s; c->seed_valid = true;
+  }
+  const int S = (int)live.size();
+  int rc;
+  if ((rc = ensure_ws(c, S)) || (rc = meta_host_free(c))) return rc;
+  const MetaPtrs hp = meta_layout(sm->meta_host, S, S, S), dp = meta_layout(sm->meta_dev, S, S, S);
+  for (int e = 0; e < S; e++) {
+    const int r = live[(size_t)e];
+    assign_pages(sm, r, c->row_past[(size_t)r] + n);
+    hp.ent_row[e] = r; hp.ent_start[e] = e; hp.ent_count[e] = 1; hp.ent_par[e] = sm->row_par[(size_t)r];
+    hp.tok_id[e] = 0; hp.tok_pos[e] = (int)c->row_past[(size_t)r]; hp.tok_ent[e] = e; hp.want[e] = e; hp.want_row[e] = r;
+  }
+  if ((rc = push_tables(c)) || (rc = push_meta(c, hp.n))) return rc;
+  for (int b = 0; b < c->batch; b++) { c->row_probs_cfg[(size_t)b] = cfg; c->row_probs_ok[(size_t)b] = is_greedy(&cfg) ? 0 : 1; }
+  c->have_probs = !is_greedy(&cfg);
+  for (int s = 0; s < n; s++) {
+    hipLaunchKernelGGL(tgx::stack_gather_tok_kernel, dim3((S + 63) / 64), dim3(64), 0, c->stream, dp.tok_id, dp.ent_row, c->slab_tok, S);
+    if ((rc = run_layers(c, dp, S, S, max_keys + s + 1))) return rc;
+    run_logits(c, dp.want, S, c->slab_logits, dp.want_row);
+    for (int r : live) launch_argmax_partials(c, c->rows[(size_t)r].logits, d.vocab, c->rows[(size_t)r].part_val, c->rows[(size_t)r].part_idx);
+    launch_sample(c, 0, c->batch, cfg, /*advance_pos=*/true, /*log_step=*/true);
+    hipLaunchKernelGGL(tgx::stack_advance_kernel, dim3((S + 63) / 64), dim3(64), 0, c->stream, dp.tok_pos, dp.ent_par, S);
+    c->steps_issued++;
+  }
+  HIP_OK(c, hipGetLastError());
+  for (int r : live) { c->row_past[(size_t)r] += n; if (n & 1) sm->row_par[(size_t)r] ^= 1; }
+  refresh_rows(c);
+  c->have_logits = true;
+  return TGX_OK;
+}
+
+// the cached latents of (slot, layer) as fp32 [past][kv_rank] — test / diagnostic use
+int stack_read_latent(tgx_ctx* c, int row, int layer, float* out) {
+  StackModel* sm = c->stack;
+  if (row < 0 || row >= sm->d.max_seqs || layer < 0 || layer >= sm->d.layers || !out) return set_err(c, TGX_ERR_INVALID, "read_kv: row / layer out of range");
+  HIP_OK(c, hipStreamSynchronize(c->stream));
+  const StackLayerW& w = sm->L[(size_t)layer];
+  const size_t R = (size_t)w.d.kv_rank;
+  std::vector<unsigned char> buf(R * c->esz);
+  for (int64_t t = 0; t < c->row_past[(size_t)row]; t++) {
+    const size_t page = (size_t)sm->tbl_host[(size_t)row * sm->tbl_stride + (size_t)(t >> sm->page_shift)];
+    HIP_OK(c, hipMemcpy(buf.data(), w.pool + ((page << sm->page_shift) + (size_t)(t & (sm->page - 1))) * R * c->esz, R * c->esz, hipMemcpyDeviceToHost));
+    const std::vector<float> f = to_f32(buf.data(), (int64_t)R, c->d.compute_dtype);
+    memcpy(out + (size_t)t * R, f.data(), R * 4);
+  }
+  return TGX_OK;
+}
+
+// HBM bytes one decoded token streams at context T: every matrix the step touches (the chosen experts only) and the cached latents
+int64_t stack_bytes_per_token(const tgx_ctx* c, int64_t T) {
+  const StackModel* sm = c->stack;
+  const int64_t W = sm->d.width, es = (int64_t)c->esz;
+  int64_t b = (int64_t)sm->d.vocab * W * es;
+  for (const auto& w : sm->L) {
+    const tgx_layer_desc& l = w.d;
+    const int64_t H = l.heads, qd = H * l.dim, R = l.kv_rank, vd = H * l.vdim;
+    b += ((qd + R + vd) * W + qd * R + vd * R + W * vd) * es + T * R * es;
+    if (l.mlp == TGX_MLP_MOE) b += (int64_t)l.experts * W * 4 + (int64_t)l.top * 3 * l.ff * W * es;
+  }
+  return b;
+}

@@ -198,9 +198,13 @@ def desc_from_hf_config(cfg: dict, compute_dtype: str = "bf16", max_batch: int =
     return d
 
 
-def load_desc(model_dir: str, compute_dtype: str = "bf16", max_batch: int = 1) -> ModelDesc:
+def load_desc(model_dir: str, compute_dtype: str = "bf16", max_batch: int = 1, **stack_kw):
+    """the model class by config.json: "model_type" names a flat family (ModelDesc), "architecture" a layered one (StackDesc; stack_kw = max_ctx, budget_tokens)"""
     with open(os.path.join(model_dir, "config.json")) as f:
-        return desc_from_hf_config(json.load(f), compute_dtype, max_batch)
+        cfg = json.load(f)
+    if is_stack_config(cfg):
+        return stack_desc_from_config(cfg, compute_dtype, max_seqs=max_batch, **stack_kw)
+    return desc_from_hf_config(cfg, compute_dtype, max_batch)
 
 
 # ---- the public HF hyper-parameters of BASELINE.json's configs (SURVEY.md §8 header) --------
@@ -261,3 +265,126 @@ def known_desc(key: str, compute_dtype: str | None = None, max_batch: int = 1) -
     if compute_dtype is None:
         compute_dtype = "fp32" if cfg["model_type"] == "gpt2" else "bf16"
     return desc_from_hf_config(cfg, compute_dtype, max_batch)
+
+
+# ---- layered models (include/tgx.h tgx_stack_desc / tgx_layer_desc) -------------------------------------------------------------
+FAMILY_ZAKUSUN = 6
+MIXER_BY_NAME = {"latent_attention": 1}
+MLP_BY_NAME = {None: 0, "moe": 1}
+
+
+class CLayerDesc(ctypes.Structure):
+    """ctypes image of ``struct tgx_layer_desc``."""
+    _fields_ = [("mixer", ctypes.c_int32), ("heads", ctypes.c_int32), ("dim", ctypes.c_int32), ("vdim", ctypes.c_int32),
+                ("kv_rank", ctypes.c_int32), ("scale", ctypes.c_float), ("mlp", ctypes.c_int32), ("experts", ctypes.c_int32),
+                ("top", ctypes.c_int32), ("ff", ctypes.c_int32), ("limit", ctypes.c_float)]
+
+
+class CStackDesc(ctypes.Structure):
+    """ctypes image of ``struct tgx_stack_desc``."""
+    _fields_ = [("family", ctypes.c_int32), ("width", ctypes.c_int32), ("layers", ctypes.c_int32), ("vocab", ctypes.c_int32),
+                ("compute_dtype", ctypes.c_int32), ("max_seqs", ctypes.c_int32), ("max_ctx", ctypes.c_int32),
+                ("budget_tokens", ctypes.c_int32), ("page_tokens", ctypes.c_int32), ("norm_groups", ctypes.c_int32),
+                ("norm_eps", ctypes.c_float), ("canon_taps", ctypes.c_int32), ("logit_scale", ctypes.c_float)]
+
+
+@dataclass
+class LayerDesc:
+    mixer: str = "latent_attention"
+    heads: int = 0
+    dim: int = 0
+    vdim: int = 0
+    kv_rank: int = 0
+    scale: float = 1.0
+    mlp: "str | None" = None      # None: the layer has no feed-forward
+    experts: int = 0
+    top: int = 0
+    ff: int = 0
+    limit: float = 0.0
+
+    def to_c(self) -> CLayerDesc:
+        return CLayerDesc(MIXER_BY_NAME[self.mixer], self.heads, self.dim, self.vdim, self.kv_rank, self.scale,
+                          MLP_BY_NAME[self.mlp], self.experts, self.top, self.ff, self.limit)
+
+
+@dataclass
+class StackDesc:
+    """A model described layer by layer (Zakusun): the Python mirror of tgx_stack_desc + its tgx_layer_desc array."""
+    family: str = "zakusun"
+    width: int = 0
+    vocab: int = 0
+    layers: "list[LayerDesc]" = field(default_factory=list)
+    compute_dtype: str = "bf16"
+    max_seqs: int = 4            # sequence slots
+    max_ctx: int = 4096          # longest sequence of a slot
+    budget_tokens: int = 0       # tokens of the shared latent pool (0: max_seqs * max_ctx)
+    page_tokens: int = 64
+    norm_groups: int = 1
+    norm_eps: float = 1e-6
+    canon_taps: int = 1
+    logit_scale: float = 1.0
+    name: str = ""
+
+    # the fields the flat description shares (bench / reporting code reads them)
+    @property
+    def hidden(self): return self.width
+
+    @property
+    def max_batch(self): return self.max_seqs
+
+    def to_c(self):
+        arr = (CLayerDesc * len(self.layers))(*[l.to_c() for l in self.layers])
+        sd = CStackDesc(FAMILY_ZAKUSUN, self.width, len(self.layers), self.vocab, DTYPE_BY_NAME[self.compute_dtype], self.max_seqs,
+                        self.max_ctx, self.budget_tokens, self.page_tokens, self.norm_groups, self.norm_eps, self.canon_taps,
+                        self.logit_scale)
+        return sd, arr
+
+    def tensor_shapes(self) -> "dict[str, tuple]":
+        """checkpoint name -> shape, in file order"""
+        W, out = self.width, {}
+        out["embed"] = (self.vocab, W)
+        for i, l in enumerate(self.layers):
+            p = f"l{i}."
+            out[p + "norm1"] = (W,)
+            if l.mlp:
+                out[p + "norm2"] = (W,)
+            out[p + "mix.q"] = (l.heads * l.dim, W); out[p + "mix.dkv"] = (l.kv_rank, W); out[p + "mix.dkv.norm"] = (l.kv_rank,)
+            out[p + "mix.uk"] = (l.heads * l.dim, l.kv_rank); out[p + "mix.uv"] = (l.heads * l.vdim, l.kv_rank)
+            out[p + "mix.sink"] = (l.heads,); out[p + "mix.g"] = (l.heads * l.vdim, W); out[p + "mix.o"] = (W, l.heads * l.vdim)
+            if l.mlp == "moe":
+                for e in range(l.experts):
+                    out[p + f"mlp.e{e}.gate"] = (l.ff, W); out[p + f"mlp.e{e}.up"] = (l.ff, W); out[p + f"mlp.e{e}.down"] = (W, l.ff)
+                out[p + "mlp.router"] = (l.experts, W); out[p + "mlp.router.b"] = (l.experts,)
+            if self.canon_taps > 1:
+                out[p + "canon1"] = (W, self.canon_taps)
+                if l.mlp:
+                    out[p + "canon2"] = (W, self.canon_taps)
+            out[p + "dwa"] = (i + 2,)
+        out["final.norm"] = (W,)
+        return out
+
+
+def stack_desc_from_config(cfg: dict, compute_dtype: str = "bf16", max_seqs: int = 4, max_ctx: int = 4096, budget_tokens: int = 0) -> StackDesc:
+    """config.json of a layered model ("architecture": "Zakusun") -> StackDesc.  Every size and constant comes from the file."""
+    if cfg.get("architecture") != "Zakusun":
+        raise ValueError(f"Unsupported architecture: {cfg.get('architecture')!r}")
+    layers = []
+    for i, l in enumerate(cfg["layers"]):
+        if l["type"] not in MIXER_BY_NAME:
+            raise ValueError(f"layer {i}: mixer {l['type']!r} is not implemented")
+        m, f = l["mixer"], l.get("mlp")
+        ld = LayerDesc(mixer=l["type"], heads=int(m["heads"]), dim=int(m["dim"]), vdim=int(m["vdim"]), kv_rank=int(m["kv_rank"]),
+                       scale=float(m["scale"]))
+        if f is not None:
+            if f.get("kind") not in MLP_BY_NAME:
+                raise ValueError(f"layer {i}: feed-forward kind {f.get('kind')!r} is not implemented")
+            ld.mlp = f["kind"]; ld.experts = int(f["router"]["experts"]); ld.top = int(f["router"]["top"])
+            ld.ff = int(f["expert"]["ff"]); ld.limit = float(f["expert"]["limit"])
+        layers.append(ld)
+    return StackDesc(width=int(cfg["width"]), vocab=int(cfg["vocab"]), layers=layers, compute_dtype=compute_dtype, max_seqs=max_seqs,
+                     max_ctx=max_ctx, budget_tokens=budget_tokens, norm_groups=int(cfg["norm"]["groups"]), norm_eps=float(cfg["norm"]["eps"]),
+                     canon_taps=int(cfg["canon"]["taps"]), logit_scale=float(cfg["logit_scale"]), name="zakusun")
+
+
+def is_stack_config(cfg: dict) -> bool:
+    return "architecture" in cfg and "model_type" not in cfg

@@ -17,7 +17,7 @@ from ctypes import POINTER, c_char_p, c_double, c_float, c_int, c_int32, c_int64
 
 import numpy as np
 
-from .desc import CDesc, ModelDesc, DTYPE_BF16, DTYPE_F32, DTYPE_F16
+from .desc import CDesc, CLayerDesc, CStackDesc, ModelDesc, StackDesc, DTYPE_BF16, DTYPE_F32, DTYPE_F16
 from . import synth
 
 HERE = os.path.dirname(os.path.abspath(__file__))
@@ -54,6 +54,8 @@ class TgxError(RuntimeError):
 ABI = {
     "device_count": (c_int, [POINTER(c_int)]),
     "create": (c_int, [POINTER(CDesc), c_int, POINTER(c_void_p)]),
+    "create_stack": (c_int, [POINTER(CStackDesc), POINTER(CLayerDesc), c_int, POINTER(c_void_p)]),
+    "step_ragged": (c_int, [c_void_p, c_int, POINTER(c_int32), POINTER(c_int32), POINTER(c_int64), c_int, POINTER(c_int32), POINTER(c_float)]),
     "upload": (c_int, [c_void_p, c_char_p, c_void_p, POINTER(c_int64), c_int, c_int]),
     "finalize": (c_int, [c_void_p]),
     "destroy": (None, [c_void_p]),
@@ -142,8 +144,12 @@ class Model:
         self.be = backend or product_backend()
         self.desc = desc
         self._ctx = c_void_p()
-        cd = desc.to_c()
-        st = self.be.create(ctypes.byref(cd), device, ctypes.byref(self._ctx))
+        if isinstance(desc, StackDesc):      # a layered model (include/tgx.h tgx_create_stack)
+            sd, layers = desc.to_c()
+            st = self.be.create_stack(ctypes.byref(sd), layers, device, ctypes.byref(self._ctx))
+        else:
+            cd = desc.to_c()
+            st = self.be.create(ctypes.byref(cd), device, ctypes.byref(self._ctx))
         if st != 0:
             msg = self.be.last_error(self._ctx if self._ctx else None)
             raise TgxError(st, (msg or b"").decode())
@@ -188,6 +194,13 @@ class Model:
             self.upload(name, bits)
         return self
 
+    def load_dir(self, model_dir: str, strict: bool = False):
+        """every tensor of a model directory's checkpoint, by name (unknown keys are skipped unless strict)"""
+        from .checkpoint import iter_checkpoint
+        for name, arr in iter_checkpoint(model_dir):
+            self.upload(name, arr, strict=strict)
+        return self
+
     def load_state(self, tensors: "dict[str, np.ndarray]", strict: bool = False):
         for name, arr in tensors.items():
             self.upload(name, arr, strict=strict)
@@ -204,6 +217,21 @@ class Model:
         self._check(self.be.forward(self._ctx, ids.ctypes.data_as(POINTER(c_int64)), B, S))
         self.batch = B
         return self
+
+    def step_ragged(self, entries, want=()):
+        """one engine step over a ragged batch (layered models): entries = [(slot, token ids)], want = indices into the concatenated tokens;
+        returns their logits [len(want)][vocab]"""
+        rows = np.asarray([r for r, _ in entries], dtype=np.int32)
+        counts = np.asarray([len(t) for _, t in entries], dtype=np.int32)
+        ids = np.ascontiguousarray(np.concatenate([np.asarray(t, dtype=np.int64).reshape(-1) for _, t in entries]))
+        w = np.ascontiguousarray(np.asarray(list(want), dtype=np.int32))
+        out = np.empty((len(w), self.desc.vocab), dtype=np.float32)
+        self._check(self.be.step_ragged(self._ctx, len(rows), rows.ctypes.data_as(POINTER(c_int32)), counts.ctypes.data_as(POINTER(c_int32)),
+                                        ids.ctypes.data_as(POINTER(c_int64)), len(w), w.ctypes.data_as(POINTER(c_int32)),
+                                        out.ctypes.data_as(POINTER(c_float))))
+        if len(rows):
+            self.batch = max(self.batch, int(rows.max()) + 1)
+        return out
 
     def logits(self, rounded: bool = True) -> np.ndarray:
         out = np.empty((self.batch, self.desc.vocab), dtype=np.float32)
