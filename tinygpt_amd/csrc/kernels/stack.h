@@ -46,11 +46,11 @@ __global__ __launch_bounds__(256) void sinusoid_embed_kernel(StepMeta m, const e
 // (rows of this step where the entry holds them, the slot's state otherwise, zero before the sequence's start);
 // out = hn_t + sum_j cw[:, j] * hn_(t - taps + 1 + j).  The state (the last taps - 1 normed rows of the slot) is double-buffered per slot: this
 // step reads buffer `par` and writes buffer `par ^ 1`, so no workgroup can overwrite what another still reads.
-constexpr int CONV_MAX_TAPS = 8, NORM_MAX_GROUPS = 16;
+constexpr int CONV_MAX_TAPS = 8, NORM_MAX_GROUPS = 64;
 struct NormConvArgs {
   const float* x;        // [T][W]
   const float* nw;       // [W] norm weight
-  const float* cw;       // [W][taps] convolution weight (nullptr: no convolution, taps = 1)
+  const float* cw;       // [W][taps] convolution weight (nullptr: the norm alone)
   float* out;            // [T][W]
   float* state;          // [2][slots][taps - 1][W] for this layer and sublayer (nullptr when taps == 1)
   size_t state_buf;      // elements between the two buffers

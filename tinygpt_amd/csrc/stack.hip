@@ -346,13 +346,15 @@ int stack_create(const tgx_stack_desc* desc, const tgx_layer_desc* layers, int d
         (rc = dev_alloc(c, &w.w_ukT, qd * R * es)) || (rc = dev_alloc(c, &w.w_uv, vd * R * es)) || (rc = dev_alloc(c, &w.w_o, W * vd * es)) ||
         (rc = dev_alloc(c, &w.lat_norm, R)) || (rc = dev_alloc(c, &w.sink, H))) return rc;
     for (const char* n : {"norm1", "dwa", "mix.q", "mix.dkv", "mix.dkv.norm", "mix.uk", "mix.uv", "mix.sink", "mix.g", "mix.o"}) sm->missing.insert(p + n);
-    if (d.canon_taps > 1) { if ((rc = dev_alloc(c, &w.canon1, W * d.canon_taps))) return rc; sm->missing.insert(p + "canon1"); }
+    if ((rc = dev_alloc(c, &w.canon1, W * d.canon_taps))) return rc;      // (one tap: the filter still scales the sublayer's input)
+    sm->missing.insert(p + "canon1");
     if (l.mlp == TGX_MLP_MOE) {
       const size_t E = (size_t)l.experts, F = (size_t)l.ff;
       if ((rc = dev_alloc(c, &w.norm2, W)) || (rc = dev_alloc(c, &w.w_gate, E * F * W * es)) || (rc = dev_alloc(c, &w.w_up, E * F * W * es)) ||
           (rc = dev_alloc(c, &w.w_down, E * W * F * es)) || (rc = dev_alloc(c, &w.w_router, E * W)) || (rc = dev_alloc(c, &w.b_router, E))) return rc;
       for (const char* n : {"norm2", "mlp.router", "mlp.router.b"}) sm->missing.insert(p + n);
-      if (d.canon_taps > 1) { if ((rc = dev_alloc(c, &w.canon2, W * d.canon_taps))) return rc; sm->missing.insert(p + "canon2"); }
+      if ((rc = dev_alloc(c, &w.canon2, W * d.canon_taps))) return rc;
+      sm->missing.insert(p + "canon2");
       for (int e = 0; e < l.experts; e++)
         for (const char* n : {".gate", ".up", ".down"}) sm->missing.insert(p + "mlp.e" + std::to_string(e) + n);
       sm->max_top = std::max(sm->max_top, l.top); sm->max_ff = std::max(sm->max_ff, l.ff); sm->max_E = std::max(sm->max_E, l.experts);

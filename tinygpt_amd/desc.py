@@ -355,10 +355,9 @@ class StackDesc:
                 for e in range(l.experts):
                     out[p + f"mlp.e{e}.gate"] = (l.ff, W); out[p + f"mlp.e{e}.up"] = (l.ff, W); out[p + f"mlp.e{e}.down"] = (W, l.ff)
                 out[p + "mlp.router"] = (l.experts, W); out[p + "mlp.router.b"] = (l.experts,)
-            if self.canon_taps > 1:
-                out[p + "canon1"] = (W, self.canon_taps)
-                if l.mlp:
-                    out[p + "canon2"] = (W, self.canon_taps)
+            out[p + "canon1"] = (W, self.canon_taps)
+            if l.mlp:
+                out[p + "canon2"] = (W, self.canon_taps)
             out[p + "dwa"] = (i + 2,)
         out["final.norm"] = (W,)
         return out
