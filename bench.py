@@ -81,6 +81,8 @@ def parse():
     ap.add_argument("--profile-reps", type=int, default=8)
     ap.add_argument("--no-graph", action="store_true", help="eager launches (needed under rocprofv3 kernel tracing)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--layered", default=None, metavar="SIZE[,SIZE]", help="instead of the headline: prefill and decode throughput of the layered (Zakusun) design at "
+                    "layer sizes of real models (1b, 0.5b; random weights), beside a Llama-family model of the same width, depth and active parameters")
     ap.add_argument("--cpu-seconds", type=float, default=15.0, help="target CPU time of the cpu_baseline sample")
     return ap.parse_args()
 
@@ -301,8 +303,75 @@ def aggregate_tokens_per_s(world, steps, job_elapsed):
     return world * steps / job_elapsed
 
 
+# ---- --layered: the layered design beside its closest flat family at equal size --------------------------------------------------------------
+# (width, heads, head / value dim, latent rank, experts, top, expert ff) and the Llama-family layer of the same width whose gated MLP has the width of the
+# `top` active experts together: equal matrix bytes per decoded token apart from the attention projections
+LAYERED_SIZES = {
+    "1b": dict(width=2048, heads=16, dim=128, vdim=128, kv_rank=512, experts=16, top=4, ff=2048, llama=dict(heads=32, kv_heads=8, inter=8192)),
+    "0.5b": dict(width=1024, heads=8, dim=128, vdim=128, kv_rank=256, experts=8, top=2, ff=1536, llama=dict(heads=16, kv_heads=8, inter=3072)),
+}
+
+
+def layered_compare(args):
+    from tinygpt_amd.desc import LayerDesc, ModelDesc, StackDesc
+    from tinygpt_amd.ffi import GREEDY, Model
+    from tinygpt_amd import synth
+    L, V, S, ND, B = 8, 32000, args.prompt, min(args.steps, 64), 16
+    rows = []
+
+    def measure(m, layered):
+        """prefill of S tokens (median of 3), then ND decode steps at batch 1, then B sequences of S tokens decoding together"""
+        ids = synth.synth_prompt(V, S, 7)
+        pf = []
+        for _ in range(4):
+            m.reset_cache()
+            t0 = time.perf_counter()
+            if layered:
+                m.step_ragged([(0, ids)], [S - 1])
+            else:
+                m.forward(ids)
+            m.synchronize()
+            pf.append(time.perf_counter() - t0)
+        m.sample(GREEDY)
+        m.decode(4, GREEDY, fetch=False); m.synchronize()
+        t0 = time.perf_counter(); m.decode(ND, GREEDY, fetch=False); m.synchronize()
+        d1 = (time.perf_counter() - t0) / ND
+        m.reset_cache()
+        if layered:
+            m.step_ragged([(b, synth.synth_prompt(V, S, 8 + b)) for b in range(B)], [S * (b + 1) - 1 for b in range(B)])
+        else:
+            m.forward(np.stack([synth.synth_prompt(V, S, 8 + b) for b in range(B)]))
+        m.sample(GREEDY)
+        m.decode(4, GREEDY, fetch=False); m.synchronize()
+        t0 = time.perf_counter(); m.decode(ND, GREEDY, fetch=False); m.synchronize()
+        dB = (time.perf_counter() - t0) / ND
+        return dict(prefill_tok_s=S / sorted(pf[1:])[1], decode_b1_tok_s=1 / d1, decode_b16_tok_s=B / dB, decode_b1_ms=d1 * 1e3,
+                    decode_b1_gbps=m.bytes_per_token(S) / d1 / 1e9)
+
+    for key in args.layered.split(","):
+        z = LAYERED_SIZES[key]
+        ctx = S + 2 * ND + 64
+        sd = StackDesc(width=z["width"], vocab=V, compute_dtype=args.dtype, max_seqs=B, max_ctx=ctx, budget_tokens=B * (ctx + 64), norm_groups=2, norm_eps=1e-6,
+                       canon_taps=4, logit_scale=1.0, name=f"zakusun-{key}",
+                       layers=[LayerDesc(heads=z["heads"], dim=z["dim"], vdim=z["vdim"], kv_rank=z["kv_rank"], scale=z["dim"] ** -0.5, mlp="moe", experts=z["experts"],
+                                         top=z["top"], ff=z["ff"], limit=7.0) for _ in range(L)])
+        ld = ModelDesc(family="llama", hidden=z["width"], layers=L, heads=z["llama"]["heads"], kv_heads=z["llama"]["kv_heads"], head_dim=z["width"] // z["llama"]["heads"],
+                       inter=z["llama"]["inter"], vocab=V, max_ctx=ctx, tied=True, compute_dtype=args.dtype, norm_eps=1e-5, rope_theta=500000.0, max_batch=B, name=f"llama-{key}")
+        for desc, layered in ((sd, True), (ld, False)):
+            m = Model(desc).load_synthetic(1234, 0.02).finalize()
+            r = measure(m, layered)
+            m.close()
+            r["model"] = desc.name
+            rows.append(r)
+            print(json.dumps(r), file=sys.stderr, flush=True)
+    print(json.dumps({"metric": "layered_vs_flat_throughput", "unit": "tokens/s", "dtype": args.dtype, "data": "synthetic", "prompt": S, "layers": L, "vocab": V,
+                      "decode_steps": ND, "rows": rows}))
+
+
 def main():
     args = parse()
+    if args.layered:
+        return layered_compare(args)
     rank = int(os.environ.get("RANK", "0"))
     local_rank = int(os.environ.get("LOCAL_RANK", "0"))
     if "WORLD_SIZE" not in os.environ and args.gpus > 1:           # no launcher: be the launcher (replicas need no rendezvous service)

@@ -248,3 +248,80 @@ def test_long_decoding_through_forward_sample_decode():
         assert clear.mean() > 0.9
     assert m.past_length == 7 + 150
     m.close()
+
+
+# ---- the C++ host engine and the command line ---------------------------------------------------------------------------------------
+def write_stack_dir(path, d, t, cfg_extra=None):
+    """config.json + model.safetensors (bf16) of a layered model"""
+    import json
+    import struct
+    layers = []
+    for l in d.layers:
+        e = {"type": l.mixer, "mixer": {"heads": l.heads, "dim": l.dim, "vdim": l.vdim, "kv_rank": l.kv_rank, "scale": l.scale}, "mlp": None}
+        if l.mlp:
+            e["mlp"] = {"kind": l.mlp, "expert": {"ff": l.ff, "limit": l.limit}, "router": {"experts": l.experts, "top": l.top}}
+        layers.append(e)
+    cfg = {"architecture": "Zakusun", "width": d.width, "vocab": d.vocab, "logit_scale": d.logit_scale, "norm": {"eps": d.norm_eps, "groups": d.norm_groups},
+           "canon": {"taps": d.canon_taps}, "layers": layers}
+    with open(f"{path}/config.json", "w") as f:
+        json.dump(cfg, f)
+    header, blobs, at = {}, [], 0
+    for name, a in t.items():
+        bits = (a.astype(np.float32).view(np.uint32) >> 16).astype(np.uint16)      # the oracle's weights are bf16-representable
+        header[name] = {"dtype": "BF16", "shape": list(a.shape), "data_offsets": [at, at + bits.nbytes]}
+        blobs.append(bits.tobytes()); at += bits.nbytes
+    hj = json.dumps(header).encode()
+    with open(f"{path}/model.safetensors", "wb") as f:
+        f.write(struct.pack("<Q", len(hj)) + hj + b"".join(blobs))
+
+
+def test_host_engine_and_cli_generate_greedy(tmp_path):
+    import subprocess
+    from host_util import HostEngine, host_lib
+    from tinygpt_amd import build
+    d = small_desc("fp32", layers=[moe_layer(), plain_layer()])
+    t = so.random_tensors(d, 11)
+    write_stack_dir(str(tmp_path), d, t)
+    prompts = [tokens(d, 9, 1), tokens(d, 4, 2), tokens(d, 13, 3)]           # unequal lengths: no padding is fed
+    want = [oracle_greedy(d, t, p, 5) for p in prompts]
+    e = HostEngine(host_lib(), model_dir=str(tmp_path), device="mi355x", dtype=0, max_batch=4)
+    assert e.prepare(), e.error()
+    e.reconfigure(max_new=5)
+    ids, new, fin = e.generate_sync(prompts)
+    assert new == 5 and [ids[b, -5:].tolist() for b in range(3)] == want
+    e.reconfigure(max_new=5)
+    ids2, new2, fin2, seen = e.generate_async(prompts[2])                     # streaming: forward + the ticket pipeline
+    assert ids2[-5:].tolist() == want[2]
+    e.close()
+    build.build_host()
+    arg = ";".join(",".join(str(x) for x in p) for p in prompts)
+    r = subprocess.run([build.HOST_CLI, "--model", str(tmp_path), "--dtype", "fp32", "--max-tokens", "5", "--temperature", "0", "--top-p", "1", "--prompt-ids", arg,
+                        "--context", "256"], capture_output=True, text=True, timeout=120)
+    assert r.returncode == 0, r.stderr
+    outs = [[int(x) for x in line.split(":")[1].split()] for line in r.stdout.splitlines() if line.startswith("Output ids")]
+    assert outs == want
+
+
+def test_trace_replay_script(tmp_path):
+    """bin/trace_run: steps in on stdin, logits out as files, 'done <n>' per step; slots are named by the trace's request ids"""
+    import json
+    import subprocess
+    import sys
+    d = small_desc("fp32", layers=[plain_layer(), moe_layer()])
+    t = so.random_tensors(d, 12)
+    mdir, out = tmp_path / "m", tmp_path / "o"
+    mdir.mkdir()
+    write_stack_dir(str(mdir), d, t)
+    a, b = tokens(d, 30, 1), tokens(d, 12, 2)
+    steps = [{"step": 0, "entries": [{"id": "x", "tokens": a[:20], "want": [0, 19]}], "end": []},
+             {"step": 1, "entries": [{"id": "y", "tokens": b[:11], "want": []}, {"id": "x", "tokens": a[20:22], "want": [1]}], "end": []},
+             {"step": 2, "entries": [{"id": "x", "tokens": a[22:], "want": [7]}, {"id": "y", "tokens": b[11:], "want": [0]}], "end": ["x", "y"]}]
+    root = __import__("os").path.dirname(__import__("os").path.dirname(__import__("os").path.abspath(__file__)))
+    r = subprocess.run([sys.executable, f"{root}/bin/trace_run", "--model", str(mdir), "--dtype", "float32", "--out", str(out), "--max-tokens", "128"],
+                       input="\n".join(json.dumps(s) for s in steps) + "\n", capture_output=True, text=True, timeout=300)
+    assert r.returncode == 0, r.stderr
+    assert [l for l in r.stdout.splitlines() if l.startswith("done")] == ["done 0", "done 1", "done 2"]
+    wa, wb = so.forward(d, t, a), so.forward(d, t, b)
+    check(np.fromfile(out / "0.f32", "<f4").reshape(2, -1), wa[[0, 19]], "fp32")
+    check(np.fromfile(out / "1.f32", "<f4").reshape(1, -1), wa[[21]], "fp32")
+    check(np.fromfile(out / "2.f32", "<f4").reshape(2, -1), np.stack([wa[29], wb[11]]), "fp32")

@@ -55,7 +55,7 @@ bool GPTEngine::prepare() {
     if (!known_config(config_.synthetic, config_.dtype, config_.maxBatch, model_.config)) return fail("unknown synthetic config: " + config_.synthetic);
     if (!load_synthetic(be_, model_.config, config_.deviceOrdinal, 1234, 0.02, &model_.ctx, err_)) return fail("Prepare failed: " + err_);
   } else {
-    if (!load_model_dir(be_, config_.modelDir, config_.deviceOrdinal, config_.dtype, config_.maxBatch, model_, err_)) return fail("Prepare failed: " + err_);
+    if (!load_model_dir(be_, config_.modelDir, config_.deviceOrdinal, config_.dtype, config_.maxBatch, model_, err_, config_.maxContext, config_.cacheTokens)) return fail("Prepare failed: " + err_);
   }
   // tokenizer: optional for the id entry points, required for the text ones (ModelLoader.cpp:60-69 always loads it)
   const std::string tdir = !config_.tokenizerDir.empty() ? config_.tokenizerDir : config_.modelDir;
@@ -119,7 +119,24 @@ GPTOutput GPTEngine::generateSync(const std::vector<std::vector<int32_t>>& promp
 
   // prefill (mask ignored, like the reference: "TODO padding mask", GPTEngine.cpp:95)
   const auto t0 = std::chrono::steady_clock::now();
-  if (be_.forward(model_.ctx, ids.data(), B, (int)S) != TGX_OK) { fail(std::string("forward: ") + be_.last_error(model_.ctx)); return out; }
+  if (model_.config.layered) {
+    // a layered model steps ragged batches: every prompt enters at its own length, one sequence slot each, in ONE pass (no pad token is ever fed; the
+    // left padding of `ids` only keeps GPTOutput.tokenIds in the reference's layout).  Prompts longer than the slot context keep their tail.
+    if (!be_.step_ragged) { fail("generateSync: the device shim does not step ragged batches"); return out; }
+    be_.reset_cache(model_.ctx);
+    std::vector<int32_t> rows((size_t)B), counts((size_t)B), want((size_t)B);
+    std::vector<int64_t> flat;
+    for (int b = 0; b < B; b++) {
+      const auto& p = prompts[(size_t)b];
+      if (p.empty()) { fail("generateSync: an empty prompt cannot be stepped"); return out; }
+      const size_t n = std::min<size_t>(p.size(), (size_t)S), off = p.size() - n;
+      rows[(size_t)b] = b; counts[(size_t)b] = (int32_t)n;
+      for (size_t i = 0; i < n; i++) flat.push_back(p[off + i]);
+      want[(size_t)b] = (int32_t)flat.size() - 1;
+    }
+    std::vector<float> logits((size_t)B * (size_t)model_.config.desc.vocab);
+    if (be_.step_ragged(model_.ctx, B, rows.data(), counts.data(), flat.data(), B, want.data(), logits.data()) != TGX_OK) { fail(std::string("step: ") + be_.last_error(model_.ctx)); return out; }
+  } else if (be_.forward(model_.ctx, ids.data(), B, (int)S) != TGX_OK) { fail(std::string("forward: ") + be_.last_error(model_.ctx)); return out; }
   std::vector<int64_t> first((size_t)B), rest((size_t)(B * (n_new - 1)));
   if (be_.sample(model_.ctx, &sc, config_.seed, first.data()) != TGX_OK) { fail(std::string("sample: ") + be_.last_error(model_.ctx)); return out; }
   const auto t1 = std::chrono::steady_clock::now();
@@ -151,6 +168,7 @@ GPTOutput GPTEngine::generateAsync(const std::vector<int32_t>& prompt, const Gen
   if (S == 0) { fail("generateAsync: the prompt is empty (nothing to prefill)"); return out; }
   const tgx_sampler_cfg sc = to_c(config_.samplerConfig);
   const auto t0 = std::chrono::steady_clock::now();
+  if (model_.config.layered) be_.reset_cache(model_.ctx);      // slot 0 starts a new sequence (a layered model's forward continues whatever the slot holds)
   if (be_.forward(model_.ctx, ids.data(), 1, (int)S) != TGX_OK) { fail(std::string("forward: ") + be_.last_error(model_.ctx)); return out; }
   int64_t cur = 0;
   if (be_.sample(model_.ctx, &sc, config_.seed, &cur) != TGX_OK) { fail(std::string("sample: ") + be_.last_error(model_.ctx)); return out; }

@@ -35,6 +35,8 @@ struct GPTConfig {       // src/engine/GPTEngine.h:25-32 (+ where to find the de
   int maxBatch = 4;
   uint64_t seed = 0;
   std::string tokenizerDir;          // tokenizer.json + tokenizer_config.json; default: modelDir (lets --synthetic runs take text)
+  int maxContext = 0;                // layered models: tokens a sequence slot may hold (0: 4096); the flat families read theirs from config.json
+  int cacheTokens = 0;               // layered models: tokens of the cache pool the slots share (0: maxBatch * maxContext)
 #ifdef TGXH_TEST_HOOKS
   // Only in the test build (tests/_build/libtgx_host_test.so, tgx_cli_test: -DTGXH_TEST_HOOKS): bind another library that exports the tgx ABI
   // (the CPU oracle) to check host logic without a GPU.  The shipped library and CLI do not contain these fields or the code that reads them:

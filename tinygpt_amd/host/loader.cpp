@@ -52,12 +52,61 @@ static bool check_dims(const tgx_model_desc& d, const std::string& path, std::st
   return true;
 }
 
-bool load_model_config(const std::string& path, int compute_dtype, int max_batch, ModelConfig& out, std::string& err) {
+// config.json of a layered model: {"architecture": "Zakusun", "width", "vocab", "logit_scale", "norm": {"eps", "groups"}, "canon": {"taps"},
+// "layers": [{"type": mixer, "mixer": {heads, dim, vdim, kv_rank, scale}, "mlp": null | {"kind": "moe", "expert": {ff, limit}, "router": {experts, top}}}]}
+static bool load_stack_config(const Json& doc, const std::string& path, int compute_dtype, int max_batch, int max_ctx, int budget_tokens, ModelConfig& out, std::string& err) {
+  const std::string arch = doc.get_str("architecture", "");
+  if (arch != "Zakusun") { err = "Unsupported architecture: " + arch; return false; }
+  auto dim = [](const Json& j, const char* key) -> int32_t { const int64_t v = j.get_int(key, -1); return (v < 0 || v > ((int64_t)1 << 30)) ? -1 : (int32_t)v; };
+  out.layered = true;
+  out.model_type = "zakusun";
+  tgx_stack_desc& s = out.stack;
+  s.family = TGX_FAMILY_ZAKUSUN;
+  s.width = dim(doc, "width"); s.vocab = dim(doc, "vocab"); s.compute_dtype = compute_dtype;
+  s.max_seqs = max_batch < 1 ? 1 : max_batch;
+  s.max_ctx = max_ctx > 0 ? max_ctx : 4096;
+  s.budget_tokens = budget_tokens > 0 ? budget_tokens : 0;
+  s.page_tokens = 0;
+  s.logit_scale = doc.get_float("logit_scale", 1.f);
+  const Json* norm = doc.get("norm");
+  const Json* canon = doc.get("canon");
+  const Json* layers = doc.get("layers");
+  if (!norm || norm->kind != Json::Obj || !canon || canon->kind != Json::Obj || !layers || layers->kind != Json::Arr || layers->arr.empty()) {
+    err = "config.json: norm / canon / layers are missing in " + path; return false;
+  }
+  s.norm_groups = dim(*norm, "groups"); s.norm_eps = norm->get_float("eps", 1e-6f); s.canon_taps = dim(*canon, "taps");
+  for (size_t i = 0; i < layers->arr.size(); i++) {
+    const Json& L = layers->arr[i];
+    const Json* mx = L.get("mixer");
+    const Json* ff = L.get("mlp");
+    tgx_layer_desc l{};
+    const std::string type = L.get_str("type", "");
+    if (type != "latent_attention" || !mx || mx->kind != Json::Obj) { err = "config.json: layer " + std::to_string(i) + ": mixer '" + type + "' is not implemented"; return false; }
+    l.mixer = TGX_MIXER_LATENT_ATTENTION;
+    l.heads = dim(*mx, "heads"); l.dim = dim(*mx, "dim"); l.vdim = dim(*mx, "vdim"); l.kv_rank = dim(*mx, "kv_rank"); l.scale = mx->get_float("scale", 1.f);
+    if (ff && ff->kind == Json::Obj) {
+      const Json* ex = ff->get("expert");
+      const Json* ro = ff->get("router");
+      if (ff->get_str("kind", "") != "moe" || !ex || !ro) { err = "config.json: layer " + std::to_string(i) + ": feed-forward kind '" + ff->get_str("kind", "") + "' is not implemented"; return false; }
+      l.mlp = TGX_MLP_MOE;
+      l.ff = dim(*ex, "ff"); l.limit = ex->get_float("limit", 0.f); l.experts = dim(*ro, "experts"); l.top = dim(*ro, "top");
+    }
+    out.layers.push_back(l);
+  }
+  s.layers = (int32_t)out.layers.size();
+  tgx_model_desc& d = out.desc;
+  d.family = s.family; d.hidden = s.width; d.layers = s.layers; d.vocab = s.vocab; d.max_ctx = s.max_ctx; d.max_batch = s.max_seqs; d.compute_dtype = compute_dtype; d.tied = 1;
+  if (s.width <= 0 || s.vocab <= 0 || s.norm_groups <= 0 || s.canon_taps <= 0) { err = "config.json: width / vocab / norm.groups / canon.taps missing or out of range in " + path; return false; }
+  return true;
+}
+
+bool load_model_config(const std::string& path, int compute_dtype, int max_batch, ModelConfig& out, std::string& err, int max_ctx, int budget_tokens) {
   std::string text;
   if (!read_file(path, text) || text.empty()) { err = "Failed to open file: " + path; return false; }
   Json doc;
   if (!JsonParser::parse(text.data(), text.size(), doc) || doc.kind != Json::Obj) { err = "JSON parse error in: " + path; return false; }
   out = ModelConfig();
+  if (!doc.has("model_type") && doc.has("architecture")) return load_stack_config(doc, path, compute_dtype, max_batch, max_ctx, budget_tokens, out, err);
   out.model_type = doc.get_str("model_type", "");
   if (out.model_type.empty()) { err = "Missing or invalid model_type in config.json"; return false; }
   const int fam = family_of(out.model_type);
@@ -218,10 +267,13 @@ bool load_safetensors(const Backend& be, tgx_ctx* ctx, const std::string& path, 
 }
 
 bool load_model_dir(const Backend& be, const std::string& dir, int device_ordinal, int compute_dtype, int max_batch,
-                    LoadedModel& out, std::string& err) {
-  if (!load_model_config(join_path(dir, "config.json"), compute_dtype, max_batch, out.config, err)) return false;
-  if (!load_generation_config(join_path(dir, "generation_config.json"), out.generation, err)) return false;   // required (ModelLoader.cpp:34-38)
-  int rc = be.create(&out.config.desc, device_ordinal, &out.ctx);
+                    LoadedModel& out, std::string& err, int max_ctx, int budget_tokens) {
+  if (!load_model_config(join_path(dir, "config.json"), compute_dtype, max_batch, out.config, err, max_ctx, budget_tokens)) return false;
+  if (out.config.layered) {      // generation_config.json is optional for a layered model (no HF export defines one)
+    if (file_exists(join_path(dir, "generation_config.json")) && !load_generation_config(join_path(dir, "generation_config.json"), out.generation, err)) return false;
+    if (!be.create_stack) { err = "the device shim does not provide layered models (tgx_create_stack)"; return false; }
+  } else if (!load_generation_config(join_path(dir, "generation_config.json"), out.generation, err)) return false;   // required (ModelLoader.cpp:34-38)
+  int rc = out.config.layered ? be.create_stack(&out.config.stack, out.config.layers.data(), device_ordinal, &out.ctx) : be.create(&out.config.desc, device_ordinal, &out.ctx);
   if (rc != TGX_OK) { err = std::string("create failed: ") + be.last_error(out.ctx); if (out.ctx) be.destroy(out.ctx); out.ctx = nullptr; return false; }
   std::string mp = join_path(dir, "model.safetensors");
   if (!file_exists(mp)) mp = join_path(dir, "model.safetensors.index.json");          // ModelLoader.cpp:72-75

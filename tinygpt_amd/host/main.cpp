@@ -34,7 +34,9 @@ static void usage(const char* prog) {
           "  --stream                  batch-1 generateAsync: print UTF-8-safe chunks as they are produced\n"
           "  --prompt-ids <a,b,c;d,e>  prompts as token ids, ';' between batch rows (default without a tokenizer: the 4 prompts as gpt2 ids)\n"
           "  --pad-id <n>              left-pad id (default: eos_token_id of the model, else 0)\n"
-          "  --seed <n>                sampler seed (default: 0)\n",
+          "  --seed <n>                sampler seed (default: 0)\n"
+          "  --context <n>             layered models: tokens a sequence slot may hold (default: 4096)\n"
+          "  --cache-tokens <n>        layered models: tokens of the cache pool shared by the slots (default: slots * context)\n",
           prog);
 }
 
@@ -66,6 +68,8 @@ int main(int argc, char** argv) {
     else if (a == "--stream") stream = true;
     else if (a == "--pad-id") pad_id = atol(next());
     else if (a == "--seed") cfg.seed = strtoull(next(), nullptr, 10);
+    else if (a == "--context") cfg.maxContext = atoi(next());
+    else if (a == "--cache-tokens") cfg.cacheTokens = atoi(next());
 #ifdef TGXH_TEST_HOOKS
     // tgx_cli_test only (tests/_build, -DTGXH_TEST_HOOKS): bind the host engine to a library of the test's choice that exports the tgx ABI
     // (the CPU oracle), to check host logic on a machine without a GPU.  The shipped tgx_cli has neither flag.
