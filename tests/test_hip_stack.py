@@ -325,3 +325,30 @@ def test_trace_replay_script(tmp_path):
     check(np.fromfile(out / "0.f32", "<f4").reshape(2, -1), wa[[0, 19]], "fp32")
     check(np.fromfile(out / "1.f32", "<f4").reshape(1, -1), wa[[21]], "fp32")
     check(np.fromfile(out / "2.f32", "<f4").reshape(2, -1), np.stack([wa[29], wb[11]]), "fp32")
+
+
+# ---- latent attention on the matrix cores (16-bit storage, latent widths of 128 .. 512) ---------------------------------------------
+@pytest.mark.parametrize("heads,rank", [(3, 128), (16, 256), (5, 384), (32, 128), (40, 512)])
+def test_matrix_core_attention_equals_the_lane_kernel(heads, rank):
+    """the same bf16 weights and cached latents through both attention kernels: portions whose 32-row tiles cut through tokens, a mixed batch,
+    decoding, contexts across page borders, and the split-keys form.  The two differ by summation order and the two-term rounding of q' and p only."""
+    d = small_desc("bf16", width=64, budget_tokens=2048, layers=[plain_layer(heads=heads, dim=8, vdim=8, kv_rank=rank, scale=1.5), moe_layer(heads=heads, kv_rank=rank, dim=4)])
+    t = so.random_tensors(d, heads)
+    tens = {k: v.astype(np.float32) for k, v in t.items()}
+    fast, slow = SlotEngine(desc=d, tensors=tens), SlotEngine(desc=d, tensors=tens)
+    slow.model.set_option("attn.mfma", 0)
+    a, b, c = tokens(d, 200, 1), tokens(d, 75, 2), tokens(d, 9, 3)
+    want = so.forward(d, t, a)[[0, 1, 69, 130, 131, 199]]
+    outs = []
+    for eng in (fast, slow):
+        o = [eng.step([("a", a[:70], [0, 1, 69]), ("b", b[:3], [2])])]
+        o.append(eng.step([("a", a[70:131], [60]), ("c", c, [8]), ("b", b[3:4], [0])]))
+        o.append(eng.step([("b", b[4:], [70]), ("a", a[131:132], [0])]))
+        o.append(eng.step([("a", a[132:199], [])]))
+        eng.model.set_option("attn.split_min", 64)
+        o.append(eng.step([("a", a[199:], [0]), ("b", [5], [0])]))
+        outs.append(np.concatenate(o))
+    assert np.abs(outs[0] - outs[1]).max() / np.abs(outs[1]).max() < 3e-4
+    check(outs[0][[0, 1, 2, 4, 8, 9]], want, "bf16")               # a's positions 0, 1, 69, 130, 131, 199 in the order the steps returned them
+    check(outs[0][[6, 7]], so.forward(d, t, b)[[3, 74]], "bf16")
+    fast.close(); slow.close()

@@ -105,6 +105,7 @@ struct LatentAppendArgs {
   const float* src; long long lds; int col0;     // the projection output [T][lds], latent columns from col0
   const float* nw;                               // [rank]
   void* pool;                                    // [pages][page][rank]
+  void* poolT;                                   // [pages][rank][page]: the same latents, token-contiguous per channel (nullptr: not kept)
   int rank; float eps;
 };
 template <int DT>
@@ -117,7 +118,12 @@ __global__ __launch_bounds__(64) void latent_append_kernel(StepMeta m, LatentApp
   const float rinv = 1.0f / sqrtf(ss / (float)a.rank + a.eps);
   const int page = m.tbl[(size_t)m.ent_row[e] * m.tbl_stride + (pos >> m.page_shift)];
   elem_t<DT>* dst = reinterpret_cast<elem_t<DT>*>(a.pool) + (((size_t)page << m.page_shift) + (size_t)(pos & ((1 << m.page_shift) - 1))) * a.rank;
-  for (int c = lane; c < a.rank; c += 64) dst[c] = f32_to_elem<DT>(s[c] * rinv * a.nw[c]);
+  elem_t<DT>* dstT = a.poolT ? reinterpret_cast<elem_t<DT>*>(a.poolT) + (((size_t)page * a.rank) << m.page_shift) + (size_t)(pos & ((1 << m.page_shift) - 1)) : nullptr;
+  for (int c = lane; c < a.rank; c += 64) {
+    const elem_t<DT> v = f32_to_elem<DT>(s[c] * rinv * a.nw[c]);
+    dst[c] = v;
+    if (dstT) dstT[(size_t)c << m.page_shift] = v;
+  }
 }
 
 // ---- latent attention, one workgroup per (token, head): the four waves take every fourth key, lanes hold rank / 64 latent channels each.

@@ -20,6 +20,7 @@ struct StackLayerW {
   ebyte *w_gate = nullptr, *w_up = nullptr, *w_down = nullptr;      // [experts][ff][width] x 2, [experts][width][ff]
   float *w_router = nullptr, *b_router = nullptr;                   // fp32 [experts][width], [experts]
   ebyte* pool = nullptr;        // latent cache of this layer: [pages][page_tokens][kv_rank]
+  ebyte* poolT = nullptr;       // ... and its transposed copy [pages][kv_rank][page_tokens] for the matrix-core attention (layers that take it)
   float* conv_state = nullptr;  // [2 sublayers][2 buffers][slots][taps - 1][width]
 };
 
@@ -44,6 +45,7 @@ struct StackModel {
   int *sel = nullptr, *moe_off = nullptr, *perm = nullptr, *ptok = nullptr, *tile_e = nullptr, *tile_m0 = nullptr, *n_tiles = nullptr;
   int max_in = 0, max_hr = 0, max_hv = 0, max_top = 0, max_ff = 0, max_E = 0, max_rank = 0;
   int attn_split_min_keys = 2048;      // option attn.split_min: steps of few tokens split a sequence's keys between workgroups from this context on
+  int attn_mfma = 1;                   // option attn.mfma: 0 keeps every layer on the lane-per-channel attention kernels
   int gemm_wt = 0;                     // option stack.gemm_wt: force the product's tile (1: 64 x 64, 2: 128 x 128); 0 = by the number of tiles
 };
 

@@ -12,6 +12,7 @@
 
 #include "kernels/stack.h"
 #include "kernels/stack_gemm.h"
+#include "kernels/stack_attn_mfma.h"
 
 int upload_param_ext(tgx_ctx* c, ebyte* dst, const void* host, int64_t n, int src_dtype);      // abi.hip
 
@@ -107,6 +108,21 @@ void launch_attn_t(tgx_ctx* c, const tgx::StepMeta& m, const tgx::LatentAttnArgs
   else hipLaunchKernelGGL((tgx::latent_attn_kernel<DT, 16, SPLIT>), grid, dim3(256), lds, c->stream, m, a);
 }
 
+// the matrix-core attention serves 16-bit storage, latent widths of 128 .. 512 in steps of 128, pages of a multiple of 32 tokens
+bool layer_attn_mfma(const tgx_ctx* c, const tgx_layer_desc& l) {
+  return c->dt != tgx::DT_F32 && l.kv_rank % 128 == 0 && l.kv_rank <= 512 && c->stack->page_shift >= 5;
+}
+
+template <int DT, bool SPLIT>
+void launch_attn_mfma_t(tgx_ctx* c, const tgx::StepMeta& m, const tgx::LatentMfmaArgs& a, dim3 grid) {
+  switch (a.rank / 128) {
+    case 1: hipLaunchKernelGGL((tgx::latent_attn_mfma_kernel<DT, 1, SPLIT>), grid, dim3(256), 0, c->stream, m, a); break;
+    case 2: hipLaunchKernelGGL((tgx::latent_attn_mfma_kernel<DT, 2, SPLIT>), grid, dim3(256), 0, c->stream, m, a); break;
+    case 3: hipLaunchKernelGGL((tgx::latent_attn_mfma_kernel<DT, 3, SPLIT>), grid, dim3(256), 0, c->stream, m, a); break;
+    default: hipLaunchKernelGGL((tgx::latent_attn_mfma_kernel<DT, 4, SPLIT>), grid, dim3(256), 0, c->stream, m, a); break;
+  }
+}
+
 int ensure_ws(tgx_ctx* c, int T) {
   StackModel* sm = c->stack;
   if (T <= sm->cap_tokens) return TGX_OK;
@@ -147,7 +163,7 @@ int ensure_part(tgx_ctx* c, size_t elems) {
 }
 
 // the layers of one step; meta is on the device.  max_keys: the longest context any token of the step attends (host knowledge; picks the attention form)
-int run_layers(tgx_ctx* c, const MetaPtrs& mp, int T, int S, int max_keys) {
+int run_layers(tgx_ctx* c, const MetaPtrs& mp, int T, int S, int max_keys, int max_count) {
   StackModel* sm = c->stack;
   const tgx::StepMeta m = step_meta(sm, mp, T, S);
   const int W = sm->d.width, nslots = sm->d.max_seqs, nb = sm->d.canon_taps - 1;
@@ -167,7 +183,7 @@ int run_layers(tgx_ctx* c, const MetaPtrs& mp, int T, int S, int max_keys) {
     g.A = sm->a; g.lda = W; g.B = w.w_in; g.ldb = W; g.C = sm->proj; g.ldc = nin; g.M = T; g.N = nin; g.K = W; g.scale = 1.f;
     launch_gemm(c, g, tgx::SG_STORE, 1);
     tgx::LatentAppendArgs la{};
-    la.src = sm->proj; la.lds = nin; la.col0 = qd; la.nw = w.lat_norm; la.pool = w.pool; la.rank = R; la.eps = sm->d.norm_eps;
+    la.src = sm->proj; la.lds = nin; la.col0 = qd; la.nw = w.lat_norm; la.pool = w.pool; la.poolT = w.poolT; la.rank = R; la.eps = sm->d.norm_eps;
     TGX_DT_SWITCH(c->dt, hipLaunchKernelGGL(tgx::latent_append_kernel<DT>, dim3(T), dim3(64), 0, c->stream, m, la))
     // queries into latent space, head by head: ql[t][h] = scale * q[t][h] . ukT[h]^T
     g = tgx::StackGemmArgs{};
@@ -176,6 +192,29 @@ int run_layers(tgx_ctx* c, const MetaPtrs& mp, int T, int S, int max_keys) {
     launch_gemm(c, g, tgx::SG_STORE, H);
     tgx::LatentAttnArgs aa{};
     aa.q = sm->ql; aa.ldq = (long long)H * R; aa.pool = w.pool; aa.sink = w.sink; aa.out = sm->lat; aa.ldo = (long long)H * R; aa.rank = R; aa.heads = H;
+    if (w.poolT && sm->attn_mfma) {
+      // rows = (token, head) pairs of an entry in tiles of 32; few tiles and a long context: the keys are divided between workgroups
+      tgx::LatentMfmaArgs ma{};
+      ma.q = sm->ql; ma.pool = w.pool; ma.poolT = w.poolT; ma.sink = w.sink; ma.out = sm->lat; ma.rank = R; ma.heads = H; ma.terms = c->act16 ? 1 : 2;
+      const int tiles = (max_count * H + 31) / 32;
+      int nsplit = 1;
+      if (max_keys >= sm->attn_split_min_keys && (long long)tiles * S < c->num_cus) {
+        nsplit = (int)std::min<long long>(64, (2LL * c->num_cus) / ((long long)tiles * S));
+        const int per = std::max(128, ((max_keys + nsplit - 1) / nsplit + 63) / 64 * 64);
+        nsplit = (max_keys + per - 1) / per;
+        ma.keys_per = per;
+      }
+      if (nsplit > 1) {
+        int rc = ensure_part(c, (size_t)T * H * nsplit * (size_t)(R + 2));
+        if (rc) return rc;
+        ma.part = sm->part; ma.nsplit = nsplit;
+        aa.part = sm->part; aa.nsplit = nsplit;
+        if (c->dt == tgx::DT_F16) launch_attn_mfma_t<tgx::DT_F16, true>(c, m, ma, dim3(tiles, S, nsplit)); else launch_attn_mfma_t<tgx::DT_BF16, true>(c, m, ma, dim3(tiles, S, nsplit));
+        hipLaunchKernelGGL(tgx::latent_attn_merge_kernel, dim3(T, H), dim3(256), 0, c->stream, aa);
+      } else {
+        if (c->dt == tgx::DT_F16) launch_attn_mfma_t<tgx::DT_F16, false>(c, m, ma, dim3(tiles, S)); else launch_attn_mfma_t<tgx::DT_BF16, false>(c, m, ma, dim3(tiles, S));
+      }
+    } else {
     int nsplit = 1;
     if (max_keys >= sm->attn_split_min_keys && (long long)T * H < 2LL * c->num_cus) {
       nsplit = (int)std::min<long long>(64, (4LL * c->num_cus) / ((long long)T * H));
@@ -191,6 +230,7 @@ int run_layers(tgx_ctx* c, const MetaPtrs& mp, int T, int S, int max_keys) {
       hipLaunchKernelGGL(tgx::latent_attn_merge_kernel, dim3(T, H), dim3(256), 0, c->stream, aa);
     } else {
       TGX_DT_SWITCH(c->dt, (launch_attn_t<DT, false>(c, m, aa, dim3(T, H))))
+    }
     }
     // o[t][h] = (lat[t][h] . uv[h]^T) * sigmoid(gate)
     g = tgx::StackGemmArgs{};
@@ -456,6 +496,10 @@ int stack_finalize(tgx_ctx* c) {
     const size_t pe = (size_t)sm->n_pages * sm->page * (size_t)w.d.kv_rank * c->esz;
     if ((rc = dev_alloc(c, &w.pool, pe))) return rc;
     HIP_OK(c, hipMemset(w.pool, 0, pe));
+    if (layer_attn_mfma(c, w.d)) {
+      if ((rc = dev_alloc(c, &w.poolT, pe))) return rc;
+      HIP_OK(c, hipMemset(w.poolT, 0, pe));
+    }
     if (nb > 0) {
       const size_t se = 4 * B * nb * W;
       if ((rc = dev_alloc(c, &w.conv_state, se))) return rc;
@@ -501,7 +545,7 @@ void stack_destroy(tgx_ctx* c) {
   auto fr = [](void* p) { if (p) (void)hipFree(p); };
   for (auto& w : sm->L) {
     fr(w.norm1); fr(w.norm2); fr(w.canon1); fr(w.canon2); fr(w.dwa); fr(w.w_in); fr(w.w_ukT); fr(w.w_uv); fr(w.w_o); fr(w.lat_norm); fr(w.sink);
-    fr(w.w_gate); fr(w.w_up); fr(w.w_down); fr(w.w_router); fr(w.b_router); fr(w.pool); fr(w.conv_state);
+    fr(w.w_gate); fr(w.w_up); fr(w.w_down); fr(w.w_router); fr(w.b_router); fr(w.pool); fr(w.poolT); fr(w.conv_state);
   }
   fr(sm->final_norm); fr(sm->freq); fr(sm->tbl_dev); fr(sm->meta_dev); fr(sm->x); fr(sm->xs); fr(sm->a); fr(sm->proj); fr(sm->ql); fr(sm->lat); fr(sm->o); fr(sm->selw);
   fr(sm->yh); fr(sm->yd); fr(sm->xn); fr(sm->lg); fr(sm->part); fr(sm->sel); fr(sm->moe_off); fr(sm->perm); fr(sm->ptok); fr(sm->tile_e); fr(sm->tile_m0); fr(sm->n_tiles);
@@ -532,7 +576,7 @@ int stack_step(tgx_ctx* c, int S, const int32_t* rows, const int32_t* counts, co
   const tgx_stack_desc& d = sm->d;
   if (S < 1 || S > d.max_seqs || !rows || !counts || !ids || n_want < 0 || (n_want > 0 && (!want || !out_logits))) return set_err(c, TGX_ERR_INVALID, "step: bad argument");
   long long T = 0, need_pages = 0;
-  int max_keys = 0;
+  int max_keys = 0, max_count = 0;
   std::vector<char> seen((size_t)d.max_seqs, 0);
   for (int e = 0; e < S; e++) {
     const int r = rows[e];
@@ -543,6 +587,7 @@ int stack_step(tgx_ctx* c, int S, const int32_t* rows, const int32_t* counts, co
     if (after > d.max_ctx) return set_err(c, TGX_ERR_CONTEXT, "context size exceeded: slot %d would hold %lld tokens (contextSize %d)", r, after, d.max_ctx);
     need_pages += std::max<long long>(0, (after + sm->page - 1) / sm->page - sm->row_pages[(size_t)r]);
     max_keys = std::max<int>(max_keys, (int)after);
+    max_count = std::max<int>(max_count, counts[e]);
     T += counts[e];
   }
   if (T > (1 << 24)) return set_err(c, TGX_ERR_INVALID, "step: %lld tokens", T);
@@ -568,7 +613,7 @@ int stack_step(tgx_ctx* c, int S, const int32_t* rows, const int32_t* counts, co
     for (int e = 0; e < S; e++) if (want[i] == hp.ent_start[e] + counts[e] - 1) last_want[(size_t)e] = i;
   }
   if ((rc = push_tables(c)) || (rc = push_meta(c, hp.n))) return rc;
-  if ((rc = run_layers(c, dp, (int)T, S, max_keys))) return rc;
+  if ((rc = run_layers(c, dp, (int)T, S, max_keys, max_count))) return rc;
   if (n_want > 0) {
     run_logits(c, dp.want, n_want, sm->lg, nullptr);
     HIP_OK(c, hipMemcpyAsync(out_logits, sm->lg, (size_t)n_want * d.vocab * 4, hipMemcpyDeviceToHost, c->stream));
@@ -635,7 +680,7 @@ int stack_decode(tgx_ctx* c, const tgx_sampler_cfg& cfg, uint64_t seed, int n) {
   c->have_probs = !is_greedy(&cfg);
   for (int s = 0; s < n; s++) {
     hipLaunchKernelGGL(tgx::stack_gather_tok_kernel, dim3((S + 63) / 64), dim3(64), 0, c->stream, dp.tok_id, dp.ent_row, c->slab_tok, S);
-    if ((rc = run_layers(c, dp, S, S, max_keys + s + 1))) return rc;
+    if ((rc = run_layers(c, dp, S, S, max_keys + s + 1, 1))) return rc;
     run_logits(c, dp.want, S, c->slab_logits, dp.want_row);
     for (int r : live) launch_argmax_partials(c, c->rows[(size_t)r].logits, d.vocab, c->rows[(size_t)r].part_val, c->rows[(size_t)r].part_idx);
     launch_sample(c, 0, c->batch, cfg, /*advance_pos=*/true, /*log_step=*/true);
