@@ -352,3 +352,24 @@ def test_matrix_core_attention_equals_the_lane_kernel(heads, rank):
     check(outs[0][[0, 1, 2, 4, 8, 9]], want, "bf16")               # a's positions 0, 1, 69, 130, 131, 199 in the order the steps returned them
     check(outs[0][[6, 7]], so.forward(d, t, b)[[3, 74]], "bf16")
     fast.close(); slow.close()
+
+
+@pytest.mark.parametrize("dtype", ["fp32", "bf16"])
+def test_few_row_kernel_equals_the_matrix_core_tiles(dtype):
+    """steps of few rows stream the weights through the few-row kernel, larger ones take the matrix-core tiles: the same steps through both"""
+    d = small_desc(dtype, layers=[moe_layer(experts=6, top=3), plain_layer(), moe_layer()])
+    t = so.random_tensors(d, 21)
+    tens = {k: v.astype(np.float32) for k, v in t.items()}
+    few, tiles = SlotEngine(desc=d, tensors=tens), SlotEngine(desc=d, tensors=tens)
+    tiles.model.set_option("stack.gemv", 0)
+    a, b = tokens(d, 40, 1), tokens(d, 17, 2)
+    outs = []
+    for eng in (few, tiles):
+        o = [eng.step([("a", a[:1], [0])])]                                        # one row
+        o.append(eng.step([("a", a[1:3], [0, 1]), ("b", b[:1], [0])]))             # three rows, two slots
+        o.append(eng.step([("a", a[3:12], list(range(9))), ("b", b[1:8], [6])]))   # sixteen rows
+        o.append(eng.step([("a", a[12:], [27]), ("b", b[8:], [8])]))               # beyond: tiles in both engines
+        outs.append(np.concatenate(o))
+    assert np.abs(outs[0] - outs[1]).max() / np.abs(outs[1]).max() < (1e-5 if dtype == "fp32" else 3e-4)
+    check(outs[0][:12], so.forward(d, t, a)[:12], dtype)
+    few.close(); tiles.close()

@@ -233,3 +233,91 @@ constexpr size_t stack_gemm_lds() {
 }
 
 }  // namespace tgx
+
+namespace tgx {
+
+// ---- the same products for a FEW rows (decode steps): a weight-streaming kernel.  One wave per pair of output columns: every lane takes 8 weights of each
+// column per pass (one 16-byte load for the 16-bit dtypes) against the 8 activations of up to MR rows, fp32 FMA chains, one cross-lane sum per (row, column)
+// at the end.  Same argument block, batching (blockIdx.z), grouping (tile list with tiles of MR rows) and epilogues as stack_gemm_kernel; the activations
+// enter in fp32 (rounded to the storage dtype first under option act.round16).  Needs the vector-load alignment (K a multiple of 8).
+template <int DT, int EPI, bool DUAL, int MR>
+__global__ __launch_bounds__(256) void stack_gemv_kernel(const StackGemmArgs a) {
+  constexpr int NC = 2, NB = DUAL ? 2 : 1;
+  const int lane = threadIdx.x & 63, wv = threadIdx.x >> 6;
+  int z, mbase, mend;
+  if (a.z_off) {
+    if ((int)blockIdx.y >= *a.n_tiles) return;
+    z = a.tile_z[blockIdx.y]; mbase = a.tile_m0[blockIdx.y]; mend = min(a.z_off[z + 1], mbase + MR);
+  } else { z = blockIdx.z; mbase = blockIdx.y * MR; mend = min(a.M, mbase + MR); }
+  const int n0 = (blockIdx.x * 4 + wv) * NC;
+  if (n0 >= a.N) return;
+  const float* Ab = a.A + (size_t)z * a.a_zoff;
+  const float* arow[MR];
+#pragma unroll
+  for (int r = 0; r < MR; r++) { const int mc = min(mbase + r, mend - 1); arow[r] = Ab + (size_t)(a.a_rows ? a.a_rows[mc] : mc) * a.lda; }
+  const elem_t<DT>* wrow[NB][NC];
+#pragma unroll
+  for (int b = 0; b < NB; b++)
+#pragma unroll
+    for (int j = 0; j < NC; j++)
+      wrow[b][j] = reinterpret_cast<const elem_t<DT>*>(b ? a.B2 : a.B) + (size_t)z * a.b_zstride + (size_t)min(n0 + j, a.N - 1) * a.ldb;
+  float acc[NB][NC][MR];
+#pragma unroll
+  for (int b = 0; b < NB; b++)
+#pragma unroll
+    for (int j = 0; j < NC; j++)
+#pragma unroll
+      for (int r = 0; r < MR; r++) acc[b][j][r] = 0.f;
+  const int round16 = a.terms == 1;
+  const int nsl = a.K >> 3;                               // 8-element slices of a row
+  for (int s0 = lane; s0 < nsl; s0 += 128) {              // two slices per lane and pass: twice the loads in flight
+    const int s1 = s0 + 64;
+    const bool two = s1 < nsl;
+    Slice8<DT> w0[NB][NC], w1[NB][NC];
+#pragma unroll
+    for (int b = 0; b < NB; b++)
+#pragma unroll
+      for (int j = 0; j < NC; j++) { w0[b][j] = load_slice_nt<DT>(wrow[b][j], (size_t)s0); w1[b][j] = load_slice_nt<DT>(wrow[b][j], (size_t)(two ? s1 : s0)); }
+#pragma unroll
+    for (int r = 0; r < MR; r++) {
+      const f32x4* xp = reinterpret_cast<const f32x4*>(arow[r]);
+      f32x4 xa = xp[2 * s0], xb = xp[2 * s0 + 1], ya = xp[2 * (two ? s1 : s0)], yb = xp[2 * (two ? s1 : s0) + 1];
+#pragma unroll
+      for (int i = 0; i < 4; i++) {
+        xa[i] = round_storage_if<DT>(xa[i], round16); xb[i] = round_storage_if<DT>(xb[i], round16);
+        ya[i] = two ? round_storage_if<DT>(ya[i], round16) : 0.f; yb[i] = two ? round_storage_if<DT>(yb[i], round16) : 0.f;
+      }
+#pragma unroll
+      for (int b = 0; b < NB; b++)
+#pragma unroll
+        for (int j = 0; j < NC; j++) { acc[b][j][r] = dot8<DT>(acc[b][j][r], w0[b][j], xa, xb); acc[b][j][r] = dot8<DT>(acc[b][j][r], w1[b][j], ya, yb); }
+    }
+  }
+#pragma unroll
+  for (int b = 0; b < NB; b++)
+#pragma unroll
+    for (int j = 0; j < NC; j++)
+#pragma unroll
+      for (int r = 0; r < MR; r++) acc[b][j][r] = wave_sum(acc[b][j][r]);
+  if (lane != 0) return;
+#pragma unroll
+  for (int r = 0; r < MR; r++) {
+    const int m = mbase + r;
+    if (m >= mend) break;
+    const size_t crow = a.c_rows ? (size_t)a.c_rows[m] : (size_t)m;
+    float* cp = a.C + crow * a.ldc + (size_t)z * a.c_zoff;
+#pragma unroll
+    for (int j = 0; j < NC; j++) {
+      const int n = n0 + j;
+      if (n >= a.N) break;
+      const float v = acc[0][j][r];
+      if constexpr (EPI == SG_STORE) cp[n] = v * a.scale;
+      else if constexpr (EPI == SG_ADD) cp[n] += v;
+      else if constexpr (EPI == SG_GATE) cp[n] = v / (1.0f + expf(-a.G[crow * a.ldg + a.g_col0 + (size_t)z * a.c_zoff + n]));
+      else if constexpr (EPI == SG_EXPERT_ACT) cp[n] = expert_act(v, acc[NB - 1][j][r], a.limit);
+      else cp[n] = v * a.rw[crow];
+    }
+  }
+}
+
+}  // namespace tgx

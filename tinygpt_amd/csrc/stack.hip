@@ -66,8 +66,24 @@ void launch_gemm_t(tgx_ctx* c, const tgx::StackGemmArgs& a, dim3 grid1, dim3 gri
   if (wt == 1) { if (vec) go(std::integral_constant<int, 1>{}, std::true_type{}); else go(std::integral_constant<int, 1>{}, std::false_type{}); }
   else { if (vec) go(std::integral_constant<int, 2>{}, std::true_type{}); else go(std::integral_constant<int, 2>{}, std::false_type{}); }
 }
-// nz: batched products (blockIdx.z); grouped products pass max_tiles_1 = an upper bound of their 64-row tiles (the device-side list says how many are real)
-void launch_gemm(tgx_ctx* c, tgx::StackGemmArgs a, int epi, int nz, int grouped_rows = 0, int groups = 0) {
+template <int DT, int EPI, bool DUAL>
+void launch_gemv_t(tgx_ctx* c, const tgx::StackGemmArgs& a, dim3 grid, int mr) {
+  switch (mr) {
+    case 1: hipLaunchKernelGGL((tgx::stack_gemv_kernel<DT, EPI, DUAL, 1>), grid, dim3(256), 0, c->stream, a); break;
+    case 2: hipLaunchKernelGGL((tgx::stack_gemv_kernel<DT, EPI, DUAL, 2>), grid, dim3(256), 0, c->stream, a); break;
+    case 4: hipLaunchKernelGGL((tgx::stack_gemv_kernel<DT, EPI, DUAL, 4>), grid, dim3(256), 0, c->stream, a); break;
+    default: hipLaunchKernelGGL((tgx::stack_gemv_kernel<DT, EPI, DUAL, 8>), grid, dim3(256), 0, c->stream, a); break;
+  }
+}
+// rows per tile of a grouped product's plan (moe_plan_kernel tile_m): steps of few (token, expert) pairs stream the experts through the few-row kernel
+constexpr int GROUPED_FEW_PAIRS = 128, GROUPED_FEW_ROWS = 4, FEW_ROWS_MAX = 16;
+// (both products of the layer must be able to take it: their contraction lengths, the width and the expert width, in whole 8-element slices)
+int grouped_tile_rows(const tgx_ctx* c, int pairs, int width, int ff) {
+  return c->stack->gemv && pairs <= GROUPED_FEW_PAIRS && width % 8 == 0 && ff % 8 == 0 ? GROUPED_FEW_ROWS : 64;
+}
+
+// nz: batched products (blockIdx.z); grouped products pass the number of their rows and groups (the device-side tile list says how many tiles are real)
+void launch_gemm(tgx_ctx* c, tgx::StackGemmArgs a, int epi, int nz, int grouped_rows = 0, int groups = 0, int grouped_tile = 64) {
   const StackModel* sm = c->stack;
   if (a.M <= 0 && !a.z_off) return;
   if (a.N <= 0 || a.K <= 0) return;
@@ -75,6 +91,23 @@ void launch_gemm(tgx_ctx* c, tgx::StackGemmArgs a, int epi, int nz, int grouped_
   const int kq = c->dt == tgx::DT_F32 ? 4 : 8;
   const bool vec = a.K % kq == 0 && a.ldb % kq == 0 && a.b_zstride % kq == 0 && a.lda % 4 == 0 && a.a_zoff % 4 == 0 && ((uintptr_t)a.A % 16 == 0) && ((uintptr_t)a.B % 16 == 0) &&
                    (!a.B2 || (uintptr_t)a.B2 % 16 == 0);
+  const bool dual = epi == tgx::SG_EXPERT_ACT;
+  // few rows: the weight-streaming kernel (its loads take whole 8-element slices)
+  const bool few = sm->gemv && vec && a.K % 8 == 0 && a.ldb % 8 == 0 && a.b_zstride % 8 == 0 && (a.z_off ? grouped_tile == GROUPED_FEW_ROWS : a.M <= FEW_ROWS_MAX);
+  if (a.z_off && grouped_tile == GROUPED_FEW_ROWS && !few) { c->launch_fault = "grouped product: the plan was made for the few-row kernel, which these operands cannot take"; return; }
+  if (few) {
+    const int mr = a.z_off ? GROUPED_FEW_ROWS : (a.M <= 1 ? 1 : a.M <= 2 ? 2 : a.M <= 4 ? 4 : 8);
+    const dim3 grid((a.N + 7) / 8, a.z_off ? grouped_rows / mr + groups : (a.M + mr - 1) / mr, a.z_off ? 1 : nz);
+    TGX_DT_SWITCH(c->dt,
+      switch (epi) {
+        case tgx::SG_STORE: launch_gemv_t<DT, tgx::SG_STORE, false>(c, a, grid, mr); break;
+        case tgx::SG_ADD: launch_gemv_t<DT, tgx::SG_ADD, false>(c, a, grid, mr); break;
+        case tgx::SG_GATE: launch_gemv_t<DT, tgx::SG_GATE, false>(c, a, grid, mr); break;
+        case tgx::SG_ROWSCALE: launch_gemv_t<DT, tgx::SG_ROWSCALE, false>(c, a, grid, mr); break;
+        default: if (dual) launch_gemv_t<DT, tgx::SG_EXPERT_ACT, true>(c, a, grid, mr); break;
+      })
+    return;
+  }
   int wt;
   dim3 g1, g2;
   if (a.z_off) {      // grouped: the tile list is built for 64-row tiles
@@ -86,7 +119,6 @@ void launch_gemm(tgx_ctx* c, tgx::StackGemmArgs a, int epi, int nz, int grouped_
     wt = (size_t)g2.x * g2.y * g2.z >= (size_t)c->num_cus ? 2 : 1;
     if (sm->gemm_wt) wt = sm->gemm_wt;
   }
-  const bool dual = epi == tgx::SG_EXPERT_ACT;
   TGX_DT_SWITCH(c->dt,
     switch (epi) {
       case tgx::SG_STORE: launch_gemm_t<DT, tgx::SG_STORE, false>(c, a, g1, g2, wt, vec); break;
@@ -141,7 +173,8 @@ int ensure_ws(tgx_ctx* c, int T) {
     const size_t np = n * (size_t)sm->max_top;
     if ((rc = dev_alloc(c, &sm->selw, np)) || (rc = dev_alloc(c, &sm->sel, np)) || (rc = dev_alloc(c, &sm->perm, np)) || (rc = dev_alloc(c, &sm->ptok, np)) ||
         (rc = dev_alloc(c, &sm->yh, np * (size_t)sm->max_ff)) || (rc = dev_alloc(c, &sm->yd, np * W)) ||
-        (rc = dev_alloc(c, &sm->tile_e, np / 64 + (size_t)sm->max_E + 1)) || (rc = dev_alloc(c, &sm->tile_m0, np / 64 + (size_t)sm->max_E + 1))) return rc;
+        (rc = dev_alloc(c, &sm->tile_e, std::max<size_t>(np / 64, GROUPED_FEW_PAIRS / GROUPED_FEW_ROWS) + (size_t)sm->max_E + 1)) ||
+        (rc = dev_alloc(c, &sm->tile_m0, std::max<size_t>(np / 64, GROUPED_FEW_PAIRS / GROUPED_FEW_ROWS) + (size_t)sm->max_E + 1))) return rc;
   }
   sm->meta_cap = (size_t)5 * n + (size_t)4 * sm->d.max_seqs;
   if ((rc = dev_alloc(c, &sm->meta_dev, sm->meta_cap))) return rc;
@@ -251,19 +284,19 @@ int run_layers(tgx_ctx* c, const MetaPtrs& mp, int T, int S, int max_keys, int m
       hipLaunchKernelGGL(tgx::router_topk_kernel, dim3(T), dim3(256), 0, c->stream, ra);
       const int np = T * top;
       tgx::MoePlanArgs pa{};
-      pa.sel = sm->sel; pa.n_pairs = np; pa.E = ld.experts; pa.top = top; pa.tile_m = 64;
+      pa.sel = sm->sel; pa.n_pairs = np; pa.E = ld.experts; pa.top = top; pa.tile_m = grouped_tile_rows(c, np, W, ld.ff);
       pa.off = sm->moe_off; pa.perm = sm->perm; pa.tok = sm->ptok; pa.tile_e = sm->tile_e; pa.tile_m0 = sm->tile_m0; pa.n_tiles = sm->n_tiles;
       hipLaunchKernelGGL(tgx::moe_plan_kernel, dim3(1), dim3(1024), 0, c->stream, pa);
       // yh[n] = act(gate_e . a[tok(n)], up_e . a[tok(n)]) over the pairs grouped by expert
       g = tgx::StackGemmArgs{};
       g.A = sm->a; g.lda = W; g.a_rows = sm->ptok; g.B = w.w_gate; g.B2 = w.w_up; g.ldb = W; g.b_zstride = (long long)ld.ff * W; g.C = sm->yh; g.ldc = ld.ff;
       g.z_off = sm->moe_off; g.tile_z = sm->tile_e; g.tile_m0 = sm->tile_m0; g.n_tiles = sm->n_tiles; g.M = np; g.N = ld.ff; g.K = W; g.limit = ld.limit;
-      launch_gemm(c, g, tgx::SG_EXPERT_ACT, 1, np, ld.experts);
+      launch_gemm(c, g, tgx::SG_EXPERT_ACT, 1, np, ld.experts, pa.tile_m);
       // yd[pair] = router weight * (down_e . yh[n])
       g = tgx::StackGemmArgs{};
       g.A = sm->yh; g.lda = ld.ff; g.B = w.w_down; g.ldb = ld.ff; g.b_zstride = (long long)W * ld.ff; g.C = sm->yd; g.ldc = W; g.c_rows = sm->perm;
       g.z_off = sm->moe_off; g.tile_z = sm->tile_e; g.tile_m0 = sm->tile_m0; g.n_tiles = sm->n_tiles; g.M = np; g.N = W; g.K = ld.ff; g.rw = sm->selw;
-      launch_gemm(c, g, tgx::SG_ROWSCALE, 1, np, ld.experts);
+      launch_gemm(c, g, tgx::SG_ROWSCALE, 1, np, ld.experts, pa.tile_m);
     }
     tgx::CombineDepthArgs cd{};
     cd.x = sm->x; cd.y = sm->yd; cd.xs = sm->xs; cd.slot_stride = slot_stride; cd.dw = w.dwa; cd.W = W; cd.top = top; cd.n_res = li + 2;
@@ -628,6 +661,7 @@ int stack_step(tgx_ctx* c, int S, const int32_t* rows, const int32_t* counts, co
   }
   HIP_OK(c, hipGetLastError());
   HIP_OK(c, hipStreamSynchronize(c->stream));
+  LAUNCH_OK(c);
   for (int e = 0; e < S; e++) {
     const int r = rows[e];
     c->row_past[(size_t)r] += counts[e];
