@@ -371,5 +371,5 @@ def test_few_row_kernel_equals_the_matrix_core_tiles(dtype):
         o.append(eng.step([("a", a[12:], [27]), ("b", b[8:], [8])]))               # beyond: tiles in both engines
         outs.append(np.concatenate(o))
     assert np.abs(outs[0] - outs[1]).max() / np.abs(outs[1]).max() < (1e-5 if dtype == "fp32" else 3e-4)
-    check(outs[0][:12], so.forward(d, t, a)[:12], dtype)
+    check(outs[0][[0, 1, 2] + list(range(4, 13))], so.forward(d, t, a)[:12], dtype)      # (row 3 is b's first token)
     few.close(); tiles.close()

@@ -69,25 +69,28 @@ __global__ __launch_bounds__(256) void norm_conv_kernel(StepMeta m, NormConvArgs
     if (d > i) continue;                                  // wave-uniform: that row comes from the state (already normed) or lies before the start
     const float* xr = a.x + (size_t)(t - d) * a.W + (size_t)g * gw;
     float ss = 0.f;
-    for (int c = lane; c < gw; c += 64) ss = fmaf(xr[c], xr[c], ss);
+    if ((a.W & 3) == 0 && (gw & 3) == 0)
+      for (int c = 4 * lane; c < gw; c += 256) { const f32x4 v = *reinterpret_cast<const f32x4*>(xr + c); ss = fmaf(v[0], v[0], ss); ss = fmaf(v[1], v[1], ss); ss = fmaf(v[2], v[2], ss); ss = fmaf(v[3], v[3], ss); }
+    else
+      for (int c = lane; c < gw; c += 64) ss = fmaf(xr[c], xr[c], ss);
     ss = wave_sum(ss);
     if (lane == 0) s_rinv[d][g] = 1.0f / sqrtf(ss / (float)gw + a.eps);
   }
   __syncthreads();
   const float* st_old = a.state ? a.state + (size_t)par * a.state_buf + (size_t)row * nb * a.W : nullptr;
   float* st_new = a.state ? a.state + (size_t)(par ^ 1) * a.state_buf + (size_t)row * nb * a.W : nullptr;
-  for (int c = threadIdx.x; c < a.W; c += 256) {
+  // channel c of the token: the normed row, the filter over it and its predecessors, the new state
+  auto channel = [&](int c, float xv, float w, const float* cw) -> float {
     const int g = c / gw;
-    const float w = a.nw[c];
-    const float h0 = a.x[(size_t)t * a.W + c] * s_rinv[0][g] * w;
+    const float h0 = xv * s_rinv[0][g] * w;
     float acc = h0;
-    if (a.cw) {
-      acc = fmaf(a.cw[(size_t)c * a.taps + nb], h0, acc);
+    if (cw) {
+      acc = fmaf(cw[nb], h0, acc);
       for (int d = 1; d <= nb; d++) {                      // the row d steps back
         float hv = 0.f;
         if (d <= i) hv = a.x[(size_t)(t - d) * a.W + c] * s_rinv[d][g] * w;
         else if (pos - d >= 0) hv = st_old[(size_t)(nb - (d - i)) * a.W + c];       // state slot s holds position past - nb + s, past = pos - i
-        acc = fmaf(a.cw[(size_t)c * a.taps + (nb - d)], hv, acc);
+        acc = fmaf(cw[nb - d], hv, acc);
       }
       // the slot's new state = the last nb normed rows after this step: row i of cnt lands in slot nb - (cnt - i) ...
       const int s = nb - (cnt - i);
@@ -96,7 +99,18 @@ __global__ __launch_bounds__(256) void norm_conv_kernel(StepMeta m, NormConvArgs
       if (i == 0)
         for (int k = 0; k + cnt < nb; k++) st_new[(size_t)k * a.W + c] = (pos - (nb - cnt - k) >= 0) ? st_old[(size_t)(k + cnt) * a.W + c] : 0.f;
     }
-    a.out[(size_t)t * a.W + c] = acc;
+    return acc;
+  };
+  if ((a.W & 3) == 0 && (gw & 3) == 0) {
+    for (int c = 4 * threadIdx.x; c < a.W; c += 1024) {
+      const f32x4 xv = *reinterpret_cast<const f32x4*>(a.x + (size_t)t * a.W + c), wv4 = *reinterpret_cast<const f32x4*>(a.nw + c);
+      f32x4 o;
+#pragma unroll
+      for (int k = 0; k < 4; k++) o[k] = channel(c + k, xv[k], wv4[k], a.cw ? a.cw + (size_t)(c + k) * a.taps : nullptr);
+      *reinterpret_cast<f32x4*>(a.out + (size_t)t * a.W + c) = o;
+    }
+  } else {
+    for (int c = threadIdx.x; c < a.W; c += 256) a.out[(size_t)t * a.W + c] = channel(c, a.x[(size_t)t * a.W + c], a.nw[c], a.cw ? a.cw + (size_t)c * a.taps : nullptr);
   }
 }
 
@@ -200,64 +214,63 @@ __global__ __launch_bounds__(256) void latent_attn_kernel(StepMeta m, LatentAttn
 }
 // merges the split records of one (token, head) in split order
 __global__ __launch_bounds__(256) void latent_attn_merge_kernel(LatentAttnArgs a) {
+  __shared__ float s_f[64];
+  __shared__ float s_inv;
   const int t = blockIdx.x, h = blockIdx.y;
-  const float* rec = a.part + ((size_t)t * a.heads + h) * a.nsplit * (size_t)(a.rank + 2);
-  float M = -INFINITY;
-  for (int s = 0; s < a.nsplit; s++) M = fmaxf(M, rec[(size_t)s * (a.rank + 2)]);
-  float L = 0.f;
-  for (int s = 0; s < a.nsplit; s++) { const float ms = rec[(size_t)s * (a.rank + 2)]; L = fmaf(rec[(size_t)s * (a.rank + 2) + 1], ms == -INFINITY ? 0.f : expf(ms - M), L); }
-  const float inv = 1.0f / L;
+  const size_t rs = (size_t)(a.rank + 2);
+  const float* rec = a.part + ((size_t)t * a.heads + h) * a.nsplit * rs;
+  if (threadIdx.x < 64) {      // one wave: every split's weight exp(m_s - M) and the merged denominator
+    const int s = threadIdx.x;
+    const float ms = s < a.nsplit ? rec[(size_t)s * rs] : -INFINITY;
+    const float M = group_max<64>(ms);
+    const float f = ms == -INFINITY ? 0.f : expf(ms - M);
+    float lf = s < a.nsplit ? rec[(size_t)s * rs + 1] * f : 0.f;
+    for (int o = 1; o < 64; o <<= 1) { const float other = __shfl_up(lf, o, 64); if (s >= o) lf += other; }      // prefix sums: lane 63 holds the total in split order
+    s_f[s] = f;
+    if (s == 63) s_inv = 1.0f / lf;
+  }
+  __syncthreads();
+  const float inv = s_inv;
   float* o = a.out + (size_t)t * a.ldo + (size_t)h * a.rank;
   for (int c = threadIdx.x; c < a.rank; c += 256) {
     float v = 0.f;
-    for (int s = 0; s < a.nsplit; s++) { const float ms = rec[(size_t)s * (a.rank + 2)]; v = fmaf(rec[(size_t)s * (a.rank + 2) + 2 + c], ms == -INFINITY ? 0.f : expf(ms - M), v); }
+    for (int s = 0; s < a.nsplit; s++) v = fmaf(rec[(size_t)s * rs + 2 + c], s_f[s], v);
     o[c] = v * inv;
   }
 }
 
-// ---- router: z = Wr h + b in fp32 (one wave per expert, lanes over the width), the `top` largest (ties: the lower index), weights = softmax over them
+// ---- router: the `top` largest of z + b (z = Wr h, an fp32 product of fp32 weights; ties: the lower index), weights = softmax over them.  One wave per token.
 struct RouterArgs {
-  const float* h;        // [T][W]
-  const float* wr;       // [E][W] fp32
+  const float* z;        // [T][E] router products
   const float* br;       // [E]
   int* sel;              // [T][top]
   float* selw;           // [T][top]
-  int W, E, top;
+  int E, top;
 };
 constexpr int ROUTER_MAX_E = 1024, ROUTER_MAX_TOP = 64;
-__global__ __launch_bounds__(256) void router_topk_kernel(RouterArgs a) {
+__global__ __launch_bounds__(64) void router_topk_kernel(RouterArgs a) {
   __shared__ float s_z[ROUTER_MAX_E];
   __shared__ float s_v[ROUTER_MAX_TOP];
   __shared__ int s_i[ROUTER_MAX_TOP];
-  const int t = blockIdx.x, lane = threadIdx.x & 63, wv = threadIdx.x >> 6;
-  const float* h = a.h + (size_t)t * a.W;
-  for (int e = wv; e < a.E; e += 4) {
-    const float* w = a.wr + (size_t)e * a.W;
-    float s = 0.f;
-    for (int c = lane; c < a.W; c += 64) s = fmaf(h[c], w[c], s);
-    s = wave_sum(s);
-    if (lane == 0) s_z[e] = s + a.br[e];
+  const int t = blockIdx.x, lane = threadIdx.x;
+  // every lane owns the logits e = lane, lane + 64, ...: it alone writes, reads and retires them, so the loop needs no barrier; the butterfly leaves each
+  // pick in all lanes, lane 0 keeps the list
+  for (int e = lane; e < a.E; e += 64) s_z[e] = a.z[(size_t)t * a.E + e] + a.br[e];
+  for (int k = 0; k < a.top; k++) {
+    float bv = -INFINITY; int bi = 0x7fffffff;
+    for (int e = lane; e < a.E; e += 64) { const float v = s_z[e]; if (v > bv) { bv = v; bi = e; } }
+    for (int o = 32; o > 0; o >>= 1) {
+      const float ov = __shfl_xor(bv, o, 64); const int oi = __shfl_xor(bi, o, 64);
+      if (ov > bv || (ov == bv && oi < bi)) { bv = ov; bi = oi; }
+    }
+    if (bi < a.E && (bi & 63) == lane) s_z[bi] = -INFINITY;
+    if (lane == 0) { s_v[k] = bv; s_i[k] = bi < a.E ? bi : 0; }
   }
-  __syncthreads();
-  if (wv == 0) {
-    // every lane owns the logits e = lane, lane + 64, ...: it alone reads and retires them, so the loop needs no barrier; the butterfly leaves each
-    // pick in all lanes, lane 0 keeps the list
-    for (int k = 0; k < a.top; k++) {
-      float bv = -INFINITY; int bi = 0x7fffffff;
-      for (int e = lane; e < a.E; e += 64) { const float v = s_z[e]; if (v > bv) { bv = v; bi = e; } }
-      for (int o = 32; o > 0; o >>= 1) {
-        const float ov = __shfl_xor(bv, o, 64); const int oi = __shfl_xor(bi, o, 64);
-        if (ov > bv || (ov == bv && oi < bi)) { bv = ov; bi = oi; }
-      }
-      if (bi < a.E && (bi & 63) == lane) s_z[bi] = -INFINITY;
-      if (lane == 0) { s_v[k] = bv; s_i[k] = bi < a.E ? bi : 0; }
-    }
-    if (lane == 0) {
-      const float mx = s_v[0];            // the first pick is the largest
-      float den = 0.f;
-      for (int k = 0; k < a.top; k++) den += expf(s_v[k] - mx);
-      for (int k = 0; k < a.top; k++) { a.sel[(size_t)t * a.top + k] = s_i[k]; a.selw[(size_t)t * a.top + k] = expf(s_v[k] - mx) / den; }
-    }
+  if (lane == 0) {
+    const float mx = s_v[0];            // the first pick is the largest
+    float den = 0.f;
+    for (int k = 0; k < a.top; k++) den += expf(s_v[k] - mx);
+    for (int k = 0; k < a.top; k++) { a.sel[(size_t)t * a.top + k] = s_i[k]; a.selw[(size_t)t * a.top + k] = expf(s_v[k] - mx) / den; }
   }
 }
 
@@ -305,6 +318,25 @@ struct CombineDepthArgs {
 };
 __global__ __launch_bounds__(256) void combine_depth_kernel(CombineDepthArgs a) {
   const size_t t = blockIdx.x;
+  if ((a.W & 3) == 0) {
+    for (int c = 4 * threadIdx.x; c < a.W; c += 1024) {
+      f32x4 v = *reinterpret_cast<const f32x4*>(a.x + t * a.W + c);
+      for (int k = 0; k < a.top; k++) v += *reinterpret_cast<const f32x4*>(a.y + (t * a.top + k) * a.W + c);
+      *reinterpret_cast<f32x4*>(a.xs + (size_t)(a.n_res - 1) * a.slot_stride + t * a.W + c) = v;
+      f32x4 s = {0.f, 0.f, 0.f, 0.f};
+      for (int j = 0; j < a.n_res - 1; j++) {
+        const f32x4 r = *reinterpret_cast<const f32x4*>(a.xs + (size_t)j * a.slot_stride + t * a.W + c);
+        const float dj = a.dw[j];
+#pragma unroll
+        for (int k = 0; k < 4; k++) s[k] = fmaf(dj, r[k], s[k]);
+      }
+      const float dl = a.dw[a.n_res - 1];
+#pragma unroll
+      for (int k = 0; k < 4; k++) s[k] = fmaf(dl, v[k], s[k]);
+      *reinterpret_cast<f32x4*>(a.x + t * a.W + c) = s;
+    }
+    return;
+  }
   for (int c = threadIdx.x; c < a.W; c += 256) {
     float v = a.x[t * a.W + c];
     for (int k = 0; k < a.top; k++) v += a.y[(t * a.top + k) * a.W + c];

@@ -40,6 +40,7 @@ struct StackModel {
   int* meta_dev = nullptr; int* meta_host = nullptr; size_t meta_cap = 0;      // one block of ints: the StepMeta arrays + the wanted rows
   hipEvent_t meta_ev = nullptr; bool meta_pending = false;
   float *x = nullptr, *xs = nullptr, *a = nullptr, *proj = nullptr, *ql = nullptr, *lat = nullptr, *o = nullptr;
+  float* zr = nullptr;                 // [T][experts] router products
   float *selw = nullptr, *yh = nullptr, *yd = nullptr, *xn = nullptr, *lg = nullptr, *part = nullptr;
   size_t part_elems = 0;
   int *sel = nullptr, *moe_off = nullptr, *perm = nullptr, *ptok = nullptr, *tile_e = nullptr, *tile_m0 = nullptr, *n_tiles = nullptr;

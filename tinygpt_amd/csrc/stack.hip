@@ -83,12 +83,13 @@ int grouped_tile_rows(const tgx_ctx* c, int pairs, int width, int ff) {
 }
 
 // nz: batched products (blockIdx.z); grouped products pass the number of their rows and groups (the device-side tile list says how many tiles are real)
-void launch_gemm(tgx_ctx* c, tgx::StackGemmArgs a, int epi, int nz, int grouped_rows = 0, int groups = 0, int grouped_tile = 64) {
+void launch_gemm(tgx_ctx* c, tgx::StackGemmArgs a, int epi, int nz, int grouped_rows = 0, int groups = 0, int grouped_tile = 64, int dt = -1) {
   const StackModel* sm = c->stack;
+  if (dt < 0) dt = c->dt;      // (the router's weights are fp32 whatever the storage dtype)
   if (a.M <= 0 && !a.z_off) return;
   if (a.N <= 0 || a.K <= 0) return;
   a.terms = c->act16 ? 1 : 2;
-  const int kq = c->dt == tgx::DT_F32 ? 4 : 8;
+  const int kq = dt == tgx::DT_F32 ? 4 : 8;
   const bool vec = a.K % kq == 0 && a.ldb % kq == 0 && a.b_zstride % kq == 0 && a.lda % 4 == 0 && a.a_zoff % 4 == 0 && ((uintptr_t)a.A % 16 == 0) && ((uintptr_t)a.B % 16 == 0) &&
                    (!a.B2 || (uintptr_t)a.B2 % 16 == 0);
   const bool dual = epi == tgx::SG_EXPERT_ACT;
@@ -98,7 +99,7 @@ void launch_gemm(tgx_ctx* c, tgx::StackGemmArgs a, int epi, int nz, int grouped_
   if (few) {
     const int mr = a.z_off ? GROUPED_FEW_ROWS : (a.M <= 1 ? 1 : a.M <= 2 ? 2 : a.M <= 4 ? 4 : 8);
     const dim3 grid((a.N + 7) / 8, a.z_off ? grouped_rows / mr + groups : (a.M + mr - 1) / mr, a.z_off ? 1 : nz);
-    TGX_DT_SWITCH(c->dt,
+    TGX_DT_SWITCH(dt,
       switch (epi) {
         case tgx::SG_STORE: launch_gemv_t<DT, tgx::SG_STORE, false>(c, a, grid, mr); break;
         case tgx::SG_ADD: launch_gemv_t<DT, tgx::SG_ADD, false>(c, a, grid, mr); break;
@@ -119,7 +120,7 @@ void launch_gemm(tgx_ctx* c, tgx::StackGemmArgs a, int epi, int nz, int grouped_
     wt = (size_t)g2.x * g2.y * g2.z >= (size_t)c->num_cus ? 2 : 1;
     if (sm->gemm_wt) wt = sm->gemm_wt;
   }
-  TGX_DT_SWITCH(c->dt,
+  TGX_DT_SWITCH(dt,
     switch (epi) {
       case tgx::SG_STORE: launch_gemm_t<DT, tgx::SG_STORE, false>(c, a, g1, g2, wt, vec); break;
       case tgx::SG_ADD: launch_gemm_t<DT, tgx::SG_ADD, false>(c, a, g1, g2, wt, vec); break;
@@ -161,7 +162,7 @@ int ensure_ws(tgx_ctx* c, int T) {
   HIP_OK(c, hipStreamSynchronize(c->stream));
   auto fr = [](auto*& p) { if (p) (void)hipFree(p); p = nullptr; };
   fr(sm->x); fr(sm->xs); fr(sm->a); fr(sm->proj); fr(sm->ql); fr(sm->lat); fr(sm->o); fr(sm->selw); fr(sm->yh); fr(sm->yd); fr(sm->xn); fr(sm->lg);
-  fr(sm->sel); fr(sm->perm); fr(sm->ptok); fr(sm->tile_e); fr(sm->tile_m0); fr(sm->meta_dev);
+  fr(sm->sel); fr(sm->perm); fr(sm->ptok); fr(sm->tile_e); fr(sm->tile_m0); fr(sm->meta_dev); fr(sm->zr);
   if (sm->meta_host) { (void)hipHostFree(sm->meta_host); sm->meta_host = nullptr; }
   const int cap = std::max(T, 64);
   const size_t W = (size_t)sm->d.width, n = (size_t)cap;
@@ -171,7 +172,7 @@ int ensure_ws(tgx_ctx* c, int T) {
       (rc = dev_alloc(c, &sm->o, n * (size_t)sm->max_hv)) || (rc = dev_alloc(c, &sm->xn, n * W)) || (rc = dev_alloc(c, &sm->lg, n * (size_t)sm->d.vocab))) return rc;
   if (sm->max_top > 0) {
     const size_t np = n * (size_t)sm->max_top;
-    if ((rc = dev_alloc(c, &sm->selw, np)) || (rc = dev_alloc(c, &sm->sel, np)) || (rc = dev_alloc(c, &sm->perm, np)) || (rc = dev_alloc(c, &sm->ptok, np)) ||
+    if ((rc = dev_alloc(c, &sm->zr, n * (size_t)sm->max_E)) || (rc = dev_alloc(c, &sm->selw, np)) || (rc = dev_alloc(c, &sm->sel, np)) || (rc = dev_alloc(c, &sm->perm, np)) || (rc = dev_alloc(c, &sm->ptok, np)) ||
         (rc = dev_alloc(c, &sm->yh, np * (size_t)sm->max_ff)) || (rc = dev_alloc(c, &sm->yd, np * W)) ||
         (rc = dev_alloc(c, &sm->tile_e, std::max<size_t>(np / 64, GROUPED_FEW_PAIRS / GROUPED_FEW_ROWS) + (size_t)sm->max_E + 1)) ||
         (rc = dev_alloc(c, &sm->tile_m0, std::max<size_t>(np / 64, GROUPED_FEW_PAIRS / GROUPED_FEW_ROWS) + (size_t)sm->max_E + 1))) return rc;
@@ -279,9 +280,13 @@ int run_layers(tgx_ctx* c, const MetaPtrs& mp, int T, int S, int max_keys, int m
       top = ld.top;
       nc.nw = w.norm2; nc.cw = w.canon2; nc.state = nb > 0 ? w.conv_state + 2 * st_buf : nullptr;
       hipLaunchKernelGGL(tgx::norm_conv_kernel, dim3(T), dim3(256), 0, c->stream, m, nc);
+      // router: fp32 weights, fp32 products (nothing is rounded), then bias, top-k and the softmax over the chosen
+      g = tgx::StackGemmArgs{};
+      g.A = sm->a; g.lda = W; g.B = w.w_router; g.ldb = W; g.C = sm->zr; g.ldc = ld.experts; g.M = T; g.N = ld.experts; g.K = W; g.scale = 1.f;
+      launch_gemm(c, g, tgx::SG_STORE, 1, 0, 0, 64, tgx::DT_F32);
       tgx::RouterArgs ra{};
-      ra.h = sm->a; ra.wr = w.w_router; ra.br = w.b_router; ra.sel = sm->sel; ra.selw = sm->selw; ra.W = W; ra.E = ld.experts; ra.top = top;
-      hipLaunchKernelGGL(tgx::router_topk_kernel, dim3(T), dim3(256), 0, c->stream, ra);
+      ra.z = sm->zr; ra.br = w.b_router; ra.sel = sm->sel; ra.selw = sm->selw; ra.E = ld.experts; ra.top = top;
+      hipLaunchKernelGGL(tgx::router_topk_kernel, dim3(T), dim3(64), 0, c->stream, ra);
       const int np = T * top;
       tgx::MoePlanArgs pa{};
       pa.sel = sm->sel; pa.n_pairs = np; pa.E = ld.experts; pa.top = top; pa.tile_m = grouped_tile_rows(c, np, W, ld.ff);
@@ -581,7 +586,7 @@ void stack_destroy(tgx_ctx* c) {
     fr(w.w_gate); fr(w.w_up); fr(w.w_down); fr(w.w_router); fr(w.b_router); fr(w.pool); fr(w.poolT); fr(w.conv_state);
   }
   fr(sm->final_norm); fr(sm->freq); fr(sm->tbl_dev); fr(sm->meta_dev); fr(sm->x); fr(sm->xs); fr(sm->a); fr(sm->proj); fr(sm->ql); fr(sm->lat); fr(sm->o); fr(sm->selw);
-  fr(sm->yh); fr(sm->yd); fr(sm->xn); fr(sm->lg); fr(sm->part); fr(sm->sel); fr(sm->moe_off); fr(sm->perm); fr(sm->ptok); fr(sm->tile_e); fr(sm->tile_m0); fr(sm->n_tiles);
+  fr(sm->yh); fr(sm->yd); fr(sm->xn); fr(sm->lg); fr(sm->part); fr(sm->zr); fr(sm->sel); fr(sm->moe_off); fr(sm->perm); fr(sm->ptok); fr(sm->tile_e); fr(sm->tile_m0); fr(sm->n_tiles);
   if (sm->tbl_host) (void)hipHostFree(sm->tbl_host);
   if (sm->meta_host) (void)hipHostFree(sm->meta_host);
   if (sm->meta_ev) (void)hipEventDestroy(sm->meta_ev);
