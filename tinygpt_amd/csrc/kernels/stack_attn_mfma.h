@@ -78,19 +78,41 @@ __global__ __launch_bounds__(256) void latent_attn_mfma_kernel(StepMeta m, Laten
   const bool sinked = svalid && (!SPLIT || blockIdx.z == 0);
   float m_s = sinked ? a.sink[sr % H] : -INFINITY, l_s = sinked ? 1.f : 0.f;
 
+  // operand fetches run one phase ahead: the score operands of the NEXT key tile are requested while this tile's softmax and P C run, the P C operands
+  // (transposed page) at the top of the tile, ahead of its score products
+  auto key_rows = [&](int kt) -> const bf16_t* {
+    const size_t pg = (size_t)m.tbl[(size_t)slot * m.tbl_stride + (kt >> m.page_shift)];
+    return pool + ((pg << m.page_shift) + (kt & (page - 1)) + l31) * (size_t)a.rank + wv * RQ + 8 * half;
+  };
+  u32x4 bq[KS];
+  if (k0 < k1) {
+    const bf16_t* cp = key_rows(k0);
+#pragma unroll
+    for (int kk = 0; kk < KS; kk++) bq[kk] = *reinterpret_cast<const u32x4*>(cp + 16 * kk);
+  }
   for (int kt = k0; kt < k1; kt += 32) {
     const size_t pg = (size_t)m.tbl[(size_t)slot * m.tbl_stride + (kt >> m.page_shift)];
     const int off = kt & (page - 1);
+    u32x4 bt[NT][2];
+#pragma unroll
+    for (int t = 0; t < NT; t++) {
+      const bf16_t* tp = poolT + ((pg * a.rank + (size_t)(wv * RQ + 32 * t + l31)) << m.page_shift) + off + 8 * half;
+      bt[t][0] = *reinterpret_cast<const u32x4*>(tp); bt[t][1] = *reinterpret_cast<const u32x4*>(tp + 16);
+    }
     // 1. partial scores over this wave's channels
     f32x16 s;
 #pragma unroll
     for (int r = 0; r < 16; r++) s[r] = 0.f;
-    const bf16_t* cp = pool + ((pg << m.page_shift) + off + l31) * (size_t)a.rank + wv * RQ + 8 * half;
 #pragma unroll
     for (int kk = 0; kk < KS; kk++) {
-      const bf16x8 b = __builtin_bit_cast(bf16x8, *reinterpret_cast<const u32x4*>(cp + 16 * kk));
+      const bf16x8 b = __builtin_bit_cast(bf16x8, bq[kk]);
       s = mfma16<DT>(qh[kk], b, s);
       if (a.terms > 1) s = mfma16<DT>(ql[kk], b, s);
+    }
+    if (kt + 32 < k1) {
+      const bf16_t* cp = key_rows(kt + 32);
+#pragma unroll
+      for (int kk = 0; kk < KS; kk++) bq[kk] = *reinterpret_cast<const u32x4*>(cp + 16 * kk);
     }
 #pragma unroll
     for (int r = 0; r < 16; r++) s_part[wv][(r & 3) + 8 * (r >> 2) + 4 * half][l31] = s[r];
@@ -134,10 +156,9 @@ __global__ __launch_bounds__(256) void latent_attn_mfma_kernel(StepMeta m, Laten
     for (int t = 0; t < NT; t++) {
 #pragma unroll
       for (int r = 0; r < 16; r++) acc[t][r] *= cr[r];
-      const bf16_t* tp = poolT + ((pg * a.rank + (size_t)(wv * RQ + 32 * t + l31)) << m.page_shift) + off + 8 * half;
 #pragma unroll
       for (int kk = 0; kk < 2; kk++) {
-        const bf16x8 b = __builtin_bit_cast(bf16x8, *reinterpret_cast<const u32x4*>(tp + 16 * kk));
+        const bf16x8 b = __builtin_bit_cast(bf16x8, bt[t][kk]);
         acc[t] = mfma16<DT>(pa[kk], b, acc[t]);
         if (a.terms > 1) acc[t] = mfma16<DT>(pb[kk], b, acc[t]);
       }

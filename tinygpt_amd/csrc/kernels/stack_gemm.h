@@ -6,7 +6,7 @@
 //   grouped (experts):             blockIdx.y walks a tile list (expert, first row) built on the device (moe_plan_kernel); rows are gathered through
 //                                  a_rows and scattered through c_rows
 //   dual:                          two weight matrices against the same activation tile (an expert's gate and up projections), combined in the epilogue
-// Workgroup = 4 waves as 2 x 2, each WT x WT tiles of 32 x 32: 64 WT x 64 WT outputs per workgroup, K in steps of 32 staged through LDS with the
+// Workgroup = 4 waves as 2 x 2, each WT x WT tiles of 32 x 32: 64 WT x 64 WT outputs per workgroup, K in steps of 64 (32 for fp32 storage) staged through LDS with the
 // next step's global loads in flight under the MFMAs.  Any M, N, K: rows, columns and the K tail are masked; shapes that break the 16-byte
 // alignment of the vector loads take element loads (VEC = false).
 #pragma once
@@ -38,8 +38,9 @@ __device__ __forceinline__ float expert_act(float gate, float up, float limit) {
 
 template <int DT, int EPI, bool DUAL, int WT, bool VEC>
 __global__ __launch_bounds__(256) void stack_gemm_kernel(const StackGemmArgs a) {
-  constexpr int BM = 64 * WT, BN = 64 * WT, BK = 32;
   constexpr bool F32 = DT == DT_F32;
+  constexpr int BM = 64 * WT, BN = 64 * WT, BK = F32 ? 32 : 64;      // 16-bit tiles take 64 k per step: half the barriers, twice the bytes in flight
+  constexpr int ACH = BK / 4, BCH = F32 ? BK / 4 : BK / 8;            // 16-byte chunks per staged row
   constexpr int LDK = BK + 8;                       // 16-bit tiles: row-major, k contiguous, 16 bytes of padding
   constexpr int LDA = BM + 1, LDB = BN + 1;         // fp32 tiles: k-major
   constexpr int NB = DUAL ? 2 : 1;
@@ -72,7 +73,7 @@ __global__ __launch_bounds__(256) void stack_gemm_kernel(const StackGemmArgs a) 
 #pragma unroll
         for (int r = 0; r < 16; r++) acc[b][i][j][r] = 0.f;
 
-  // ---- staging maps.  A: chunks of 4 k (fp32) -> chunk c: row c / 8, k 4 (c % 8).  B: 16-bit chunks of 8 k -> row c / 4, k 8 (c % 4); fp32 as A.
+  // ---- staging maps.  A: chunks of 4 k (fp32) -> chunk c: row c / ACH, k 4 (c % ACH).  B: 16-bit chunks of 8 k -> row c / BCH, k 8 (c % BCH); fp32 as A.
   constexpr int AI = BM * (BK / 4) / 256;
   constexpr int BI = F32 ? BN * (BK / 4) / 256 : BN * (BK / 8) / 256;
   f32x4 ra[AI];
@@ -81,14 +82,14 @@ __global__ __launch_bounds__(256) void stack_gemm_kernel(const StackGemmArgs a) 
   size_t arow[AI];
 #pragma unroll
   for (int i = 0; i < AI; i++) {
-    const int m = mbase + (tid + 256 * i) / 8;
+    const int m = mbase + (tid + 256 * i) / ACH;
     const int mc = min(m, mend - 1);
     arow[i] = (size_t)(a.a_rows ? a.a_rows[mc] : mc) * a.lda;
   }
   auto load_tiles = [&](int k0) {
 #pragma unroll
     for (int i = 0; i < AI; i++) {
-      const int k = k0 + 4 * ((tid + 256 * i) & 7);
+      const int k = k0 + 4 * ((tid + 256 * i) % ACH);
       const float* p = Ab + arow[i] + k;
       if (VEC) ra[i] = k < a.K ? *reinterpret_cast<const f32x4*>(p) : f32x4{0.f, 0.f, 0.f, 0.f};
       else
@@ -101,14 +102,14 @@ __global__ __launch_bounds__(256) void stack_gemm_kernel(const StackGemmArgs a) 
       for (int i = 0; i < BI; i++) {
         const int c = tid + 256 * i;
         if constexpr (F32) {
-          const int n = min(n0 + c / 8, a.N - 1), k = k0 + 4 * (c & 7);
+          const int n = min(n0 + c / BCH, a.N - 1), k = k0 + 4 * (c % BCH);
           const float* p = reinterpret_cast<const float*>(Bz[b]) + (size_t)n * a.ldb + k;
           if (VEC) rbf[b * BI + i] = k < a.K ? *reinterpret_cast<const f32x4*>(p) : f32x4{0.f, 0.f, 0.f, 0.f};
           else
 #pragma unroll
             for (int e = 0; e < 4; e++) rbf[b * BI + i][e] = k + e < a.K ? p[e] : 0.f;
         } else {
-          const int n = min(n0 + c / 4, a.N - 1), k = k0 + 8 * (c & 3);
+          const int n = min(n0 + c / BCH, a.N - 1), k = k0 + 8 * (c % BCH);
           const bf16_t* p = reinterpret_cast<const bf16_t*>(Bz[b]) + (size_t)n * a.ldb + k;
           if (VEC) rbh[b * BI + i] = k < a.K ? *reinterpret_cast<const u32x4*>(p) : u32x4{0u, 0u, 0u, 0u};
           else {
@@ -123,7 +124,7 @@ __global__ __launch_bounds__(256) void stack_gemm_kernel(const StackGemmArgs a) 
   auto store_tiles = [&]() {
 #pragma unroll
     for (int i = 0; i < AI; i++) {
-      const int c = tid + 256 * i, row = c / 8, kc = c & 7;
+      const int c = tid + 256 * i, row = c / ACH, kc = c % ACH;
       if constexpr (F32) {
 #pragma unroll
         for (int e = 0; e < 4; e++) fA[(4 * kc + e) * LDA + row] = ra[i][e];
@@ -141,11 +142,11 @@ __global__ __launch_bounds__(256) void stack_gemm_kernel(const StackGemmArgs a) 
       for (int i = 0; i < BI; i++) {
         const int c = tid + 256 * i;
         if constexpr (F32) {
-          const int row = c / 8, kc = c & 7;
+          const int row = c / BCH, kc = c % BCH;
 #pragma unroll
           for (int e = 0; e < 4; e++) fB[(b * BK + 4 * kc + e) * LDB + row] = rbf[b * BI + i][e];
         } else {
-          const int row = c / 4, kc = c & 3;
+          const int row = c / BCH, kc = c % BCH;
           *reinterpret_cast<u32x4*>(sB + ((size_t)b * BN + row) * LDK + 8 * kc) = rbh[b * BI + i];
         }
       }
@@ -228,7 +229,7 @@ __global__ __launch_bounds__(256) void stack_gemm_kernel(const StackGemmArgs a) 
 
 template <int DT, bool DUAL, int WT>
 constexpr size_t stack_gemm_lds() {
-  constexpr int BM = 64 * WT, BN = 64 * WT, BK = 32, NB = DUAL ? 2 : 1;
+  constexpr int BM = 64 * WT, BN = 64 * WT, BK = DT == DT_F32 ? 32 : 64, NB = DUAL ? 2 : 1;
   return DT == DT_F32 ? (size_t)(BK * (BM + 1) + NB * BK * (BN + 1)) * 4 : (size_t)(2 * BM + NB * BN) * (BK + 8) * 2;
 }
 

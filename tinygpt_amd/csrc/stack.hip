@@ -117,7 +117,7 @@ void launch_gemm(tgx_ctx* c, tgx::StackGemmArgs a, int epi, int nz, int grouped_
   } else {
     g1 = dim3((a.N + 63) / 64, (a.M + 63) / 64, nz);
     g2 = dim3((a.N + 127) / 128, (a.M + 127) / 128, nz);
-    wt = (size_t)g2.x * g2.y * g2.z >= (size_t)c->num_cus ? 2 : 1;
+    wt = (size_t)g2.x * g2.y * g2.z >= 2 * (size_t)c->num_cus ? 2 : 1;      // the wide tile once it fills the chip twice over: fewer, larger tiles hide less latency
     if (sm->gemm_wt) wt = sm->gemm_wt;
   }
   TGX_DT_SWITCH(dt,
