@@ -77,8 +77,11 @@ __global__ __launch_bounds__(256) void norm_conv_kernel(StepMeta m, NormConvArgs
     if (lane == 0) s_rinv[d][g] = 1.0f / sqrtf(ss / (float)gw + a.eps);
   }
   __syncthreads();
-  const float* st_old = a.state ? a.state + (size_t)par * a.state_buf + (size_t)row * nb * a.W : nullptr;
-  float* st_new = a.state ? a.state + (size_t)(par ^ 1) * a.state_buf + (size_t)row * nb * a.W : nullptr;
+  // (the two state buffers, the stream and the output never overlap: without the qualifiers every state store would order the loads behind it)
+  const float* __restrict__ st_old = a.state ? a.state + (size_t)par * a.state_buf + (size_t)row * nb * a.W : nullptr;
+  float* __restrict__ st_new = a.state ? a.state + (size_t)(par ^ 1) * a.state_buf + (size_t)row * nb * a.W : nullptr;
+  const float* __restrict__ xin = a.x;
+  float* __restrict__ outp = a.out;
   // channel c of the token: the normed row, the filter over it and its predecessors, the new state
   auto channel = [&](int c, float xv, float w, const float* cw) -> float {
     const int g = c / gw;
@@ -88,7 +91,7 @@ __global__ __launch_bounds__(256) void norm_conv_kernel(StepMeta m, NormConvArgs
       acc = fmaf(cw[nb], h0, acc);
       for (int d = 1; d <= nb; d++) {                      // the row d steps back
         float hv = 0.f;
-        if (d <= i) hv = a.x[(size_t)(t - d) * a.W + c] * s_rinv[d][g] * w;
+        if (d <= i) hv = xin[(size_t)(t - d) * a.W + c] * s_rinv[d][g] * w;
         else if (pos - d >= 0) hv = st_old[(size_t)(nb - (d - i)) * a.W + c];       // state slot s holds position past - nb + s, past = pos - i
         acc = fmaf(cw[nb - d], hv, acc);
       }
@@ -102,15 +105,59 @@ __global__ __launch_bounds__(256) void norm_conv_kernel(StepMeta m, NormConvArgs
     return acc;
   };
   if ((a.W & 3) == 0 && (gw & 3) == 0) {
+    // four channels per thread.  Every load is issued unconditionally (where the row back comes from — this step, the state, nowhere — is uniform over the
+    // workgroup and only selects the address): one memory round trip instead of one per tap
     for (int c = 4 * threadIdx.x; c < a.W; c += 1024) {
-      const f32x4 xv = *reinterpret_cast<const f32x4*>(a.x + (size_t)t * a.W + c), wv4 = *reinterpret_cast<const f32x4*>(a.nw + c);
+      const int g = c / gw;
+      const f32x4 xv = *reinterpret_cast<const f32x4*>(xin + (size_t)t * a.W + c), wv4 = *reinterpret_cast<const f32x4*>(a.nw + c);
+      f32x4 hv[CONV_MAX_TAPS];
+      float cwv[4][CONV_MAX_TAPS];
+#pragma unroll
+      for (int d = 1; d < CONV_MAX_TAPS; d++) {
+        if (d > nb) continue;
+        const bool inrow = d <= i, ok = inrow || pos - d >= 0;
+        const float* p = inrow ? xin + (size_t)(t - d) * a.W + c : (ok ? st_old + (size_t)(nb - (d - i)) * a.W + c : xin + (size_t)t * a.W + c);
+        const f32x4 v = *reinterpret_cast<const f32x4*>(p);
+        const float sc = inrow ? s_rinv[d][g] : (ok ? 1.f : 0.f);
+#pragma unroll
+        for (int k = 0; k < 4; k++) hv[d][k] = inrow ? v[k] * sc * wv4[k] : v[k] * sc;
+      }
+      if (a.cw) {
+#pragma unroll
+        for (int k = 0; k < 4; k++)
+#pragma unroll
+          for (int j = 0; j < CONV_MAX_TAPS; j++) cwv[k][j] = j < a.taps ? a.cw[(size_t)(c + k) * a.taps + j] : 0.f;
+      }
       f32x4 o;
 #pragma unroll
-      for (int k = 0; k < 4; k++) o[k] = channel(c + k, xv[k], wv4[k], a.cw ? a.cw + (size_t)(c + k) * a.taps : nullptr);
-      *reinterpret_cast<f32x4*>(a.out + (size_t)t * a.W + c) = o;
+      for (int k = 0; k < 4; k++) { hv[0][k] = xv[k] * s_rinv[0][g] * wv4[k]; o[k] = hv[0][k]; }
+      if (a.cw) {
+#pragma unroll
+        for (int d = 0; d < CONV_MAX_TAPS; d++) {
+          if (d > nb) continue;
+#pragma unroll
+          for (int k = 0; k < 4; k++) {
+            float wsel = 0.f;                                // filter tap nb - d of channel c + k
+#pragma unroll
+            for (int j = 0; j < CONV_MAX_TAPS; j++) wsel = (j == nb - d) ? cwv[k][j] : wsel;
+            o[k] = fmaf(wsel, hv[d][k], o[k]);
+          }
+        }
+        const int sl = nb - (cnt - i);
+        if (sl >= 0) *reinterpret_cast<f32x4*>(st_new + (size_t)sl * a.W + c) = hv[0];
+        if (i == 0) {
+#pragma unroll
+          for (int d = 1; d < CONV_MAX_TAPS; d++) {          // an entry shorter than the state keeps the tail of the old one: old row d back -> slot nb - cnt - d
+            if (d > nb) continue;
+            const int kk = nb - cnt - d;
+            if (kk >= 0) *reinterpret_cast<f32x4*>(st_new + (size_t)kk * a.W + c) = hv[d];
+          }
+        }
+      }
+      *reinterpret_cast<f32x4*>(outp + (size_t)t * a.W + c) = o;
     }
   } else {
-    for (int c = threadIdx.x; c < a.W; c += 256) a.out[(size_t)t * a.W + c] = channel(c, a.x[(size_t)t * a.W + c], a.nw[c], a.cw ? a.cw + (size_t)c * a.taps : nullptr);
+    for (int c = threadIdx.x; c < a.W; c += 256) outp[(size_t)t * a.W + c] = channel(c, xin[(size_t)t * a.W + c], a.nw[c], a.cw ? a.cw + (size_t)c * a.taps : nullptr);
   }
 }
 

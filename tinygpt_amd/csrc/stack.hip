@@ -234,7 +234,7 @@ int run_layers(tgx_ctx* c, const MetaPtrs& mp, int T, int S, int max_keys, int m
       int nsplit = 1;
       if (max_keys >= sm->attn_split_min_keys && (long long)tiles * S < c->num_cus) {
         nsplit = (int)std::min<long long>(64, (2LL * c->num_cus) / ((long long)tiles * S));
-        const int per = std::max(128, ((max_keys + nsplit - 1) / nsplit + 63) / 64 * 64);
+        const int per = std::max(64, ((max_keys + nsplit - 1) / nsplit + 31) / 32 * 32);      // two key tiles per workgroup at least
         nsplit = (max_keys + per - 1) / per;
         ma.keys_per = per;
       }
