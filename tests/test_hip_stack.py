@@ -65,6 +65,7 @@ MECH = {
     "many_experts": dict(layers=[moe_layer(experts=70, top=6, ff=8)]),
     "tight_clamp": dict(layers=[moe_layer(limit=0.25)]),
     "ragged_sizes": dict(width=36, vocab=101, norm_groups=3, layers=[moe_layer(heads=3, dim=6, vdim=5, kv_rank=10, ff=18), plain_layer(heads=5, dim=4, vdim=3, kv_rank=7)]),
+    "odd_width": dict(width=27, vocab=53, norm_groups=3, canon_taps=3, layers=[moe_layer(heads=3, dim=5, vdim=7, kv_rank=9, ff=11, experts=3, top=2), plain_layer(heads=2, dim=3, vdim=5, kv_rank=6)]),
     "no_feed_forward_anywhere": dict(layers=[plain_layer(), plain_layer(), plain_layer()]),
     "deep": dict(layers=[moe_layer(), plain_layer()] * 4),
     "logit_scale": dict(logit_scale=3.0, layers=[plain_layer()]),

@@ -65,7 +65,10 @@ class SlotEngine:
         [n][vocab].  `end` lists the requests that are finished after this step."""
         batch, want, base = [], [], 0
         for rid, tokens, places in entries:
-            batch.append((self.admit(rid), tokens))
+            slot = self.admit(rid)
+            if len(tokens) == 0:                         # an entry that brings nothing this step only keeps (or takes) its slot
+                continue
+            batch.append((slot, tokens))
             want += [base + int(p) for p in places]
             base += len(tokens)
         out = self.model.step_ragged(batch, want) if batch else np.empty((0, self.desc.vocab), np.float32)
