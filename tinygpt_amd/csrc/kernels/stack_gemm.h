@@ -237,13 +237,16 @@ constexpr size_t stack_gemm_lds() {
 
 namespace tgx {
 
+// output columns per wave of the few-row kernel (four for eight-row tiles was measured slower: 16 rows x 8 layers at width 2048 6.6k -> 6.2k tokens/s)
+constexpr int stack_gemv_cols(int, bool) { return 2; }
+
 // ---- the same products for a FEW rows (decode steps): a weight-streaming kernel.  One wave per pair of output columns: every lane takes 8 weights of each
 // column per pass (one 16-byte load for the 16-bit dtypes) against the 8 activations of up to MR rows, fp32 FMA chains, one cross-lane sum per (row, column)
 // at the end.  Same argument block, batching (blockIdx.z), grouping (tile list with tiles of MR rows) and epilogues as stack_gemm_kernel; the activations
 // enter in fp32 (rounded to the storage dtype first under option act.round16).  Needs the vector-load alignment (K a multiple of 8).
 template <int DT, int EPI, bool DUAL, int MR>
 __global__ __launch_bounds__(256) void stack_gemv_kernel(const StackGemmArgs a) {
-  constexpr int NC = 2, NB = DUAL ? 2 : 1;
+  constexpr int NC = stack_gemv_cols(MR, DUAL), NB = DUAL ? 2 : 1;
   const int lane = threadIdx.x & 63, wv = threadIdx.x >> 6;
   int z, mbase, mend;
   if (a.z_off) {

@@ -77,6 +77,7 @@ void launch_gemv_t(tgx_ctx* c, const tgx::StackGemmArgs& a, dim3 grid, int mr) {
 }
 // rows per tile of a grouped product's plan (moe_plan_kernel tile_m): steps of few (token, expert) pairs stream the experts through the few-row kernel
 constexpr int GROUPED_FEW_PAIRS = 128, GROUPED_FEW_ROWS = 4, FEW_ROWS_MAX = 16;
+constexpr int FEW_COLS_ANY_ROWS = 64;      // a matrix of so few rows (the router's) is streamed per eight-row tile whatever the step's size: the 64-wide matrix-core tiles would stand mostly empty
 // (both products of the layer must be able to take it: their contraction lengths, the width and the expert width, in whole 8-element slices)
 int grouped_tile_rows(const tgx_ctx* c, int pairs, int width, int ff) {
   return c->stack->gemv && pairs <= GROUPED_FEW_PAIRS && width % 8 == 0 && ff % 8 == 0 ? GROUPED_FEW_ROWS : 64;
@@ -94,11 +95,12 @@ void launch_gemm(tgx_ctx* c, tgx::StackGemmArgs a, int epi, int nz, int grouped_
                    (!a.B2 || (uintptr_t)a.B2 % 16 == 0);
   const bool dual = epi == tgx::SG_EXPERT_ACT;
   // few rows: the weight-streaming kernel (its loads take whole 8-element slices)
-  const bool few = sm->gemv && vec && a.K % 8 == 0 && a.ldb % 8 == 0 && a.b_zstride % 8 == 0 && (a.z_off ? grouped_tile == GROUPED_FEW_ROWS : a.M <= FEW_ROWS_MAX);
+  const bool few = sm->gemv && vec && a.K % 8 == 0 && a.ldb % 8 == 0 && a.b_zstride % 8 == 0 && (a.z_off ? grouped_tile == GROUPED_FEW_ROWS : (a.M <= FEW_ROWS_MAX || a.N <= FEW_COLS_ANY_ROWS));
   if (a.z_off && grouped_tile == GROUPED_FEW_ROWS && !few) { c->launch_fault = "grouped product: the plan was made for the few-row kernel, which these operands cannot take"; return; }
   if (few) {
     const int mr = a.z_off ? GROUPED_FEW_ROWS : (a.M <= 1 ? 1 : a.M <= 2 ? 2 : a.M <= 4 ? 4 : 8);
-    const dim3 grid((a.N + 7) / 8, a.z_off ? grouped_rows / mr + groups : (a.M + mr - 1) / mr, a.z_off ? 1 : nz);
+    const int cols = 4 * tgx::stack_gemv_cols(mr, dual);      // per workgroup
+    const dim3 grid((a.N + cols - 1) / cols, a.z_off ? grouped_rows / mr + groups : (a.M + mr - 1) / mr, a.z_off ? 1 : nz);
     TGX_DT_SWITCH(dt,
       switch (epi) {
         case tgx::SG_STORE: launch_gemv_t<DT, tgx::SG_STORE, false>(c, a, grid, mr); break;
