@@ -19,6 +19,10 @@ struct StepMeta {          // device arrays of one step (T tokens, S entries)
   const int* tok_id;       // [T] token id
   const int* tok_pos;      // [T] position inside its sequence
   const int* tok_ent;      // [T] entry of the token
+  const int* tok_row;      // [T] its sequence slot, its index inside the entry, the entry's length and state buffer: copies of the per-entry values, so
+  const int* tok_idx;      //     that a one-workgroup-per-token kernel reads everything it needs in one round trip instead of two dependent ones
+  const int* tok_cnt;
+  const int* tok_par;
   const int* ent_row;      // [S] sequence slot
   const int* ent_start;    // [S] first token of the entry
   const int* ent_count;    // [S]
@@ -59,8 +63,8 @@ struct NormConvArgs {
 };
 __global__ __launch_bounds__(256) void norm_conv_kernel(StepMeta m, NormConvArgs a) {
   __shared__ float s_rinv[CONV_MAX_TAPS][NORM_MAX_GROUPS];
-  const int t = blockIdx.x, e = m.tok_ent[t], i = t - m.ent_start[e], cnt = m.ent_count[e], pos = m.tok_pos[t];
-  const int row = m.ent_row[e], par = m.ent_par[e];
+  const int t = blockIdx.x, i = m.tok_idx[t], cnt = m.tok_cnt[t], pos = m.tok_pos[t];
+  const int row = m.tok_row[t], par = m.tok_par[t];
   const int lane = threadIdx.x & 63, wv = threadIdx.x >> 6;
   const int gw = a.W / a.groups, nb = a.taps - 1;
   // 1 / rms of every (row back, group) pair that lives in this step: one wave per pair, lanes over the group's channels
@@ -107,6 +111,7 @@ __global__ __launch_bounds__(256) void norm_conv_kernel(StepMeta m, NormConvArgs
   if ((a.W & 3) == 0 && (gw & 3) == 0) {
     // four channels per thread.  Every load is issued unconditionally (where the row back comes from — this step, the state, nowhere — is uniform over the
     // workgroup and only selects the address): one memory round trip instead of one per tap
+#pragma unroll 2
     for (int c = 4 * threadIdx.x; c < a.W; c += 1024) {
       const int g = c / gw;
       const f32x4 xv = *reinterpret_cast<const f32x4*>(xin + (size_t)t * a.W + c), wv4 = *reinterpret_cast<const f32x4*>(a.nw + c);
@@ -171,13 +176,13 @@ struct LatentAppendArgs {
 };
 template <int DT>
 __global__ __launch_bounds__(64) void latent_append_kernel(StepMeta m, LatentAppendArgs a) {
-  const int t = blockIdx.x, lane = threadIdx.x, e = m.tok_ent[t], pos = m.tok_pos[t];
+  const int t = blockIdx.x, lane = threadIdx.x, pos = m.tok_pos[t];
   const float* s = a.src + (size_t)t * a.lds + a.col0;
   float ss = 0.f;
   for (int c = lane; c < a.rank; c += 64) ss = fmaf(s[c], s[c], ss);
   ss = wave_sum(ss);
   const float rinv = 1.0f / sqrtf(ss / (float)a.rank + a.eps);
-  const int page = m.tbl[(size_t)m.ent_row[e] * m.tbl_stride + (pos >> m.page_shift)];
+  const int page = m.tbl[(size_t)m.tok_row[t] * m.tbl_stride + (pos >> m.page_shift)];
   elem_t<DT>* dst = reinterpret_cast<elem_t<DT>*>(a.pool) + (((size_t)page << m.page_shift) + (size_t)(pos & ((1 << m.page_shift) - 1))) * a.rank;
   elem_t<DT>* dstT = a.poolT ? reinterpret_cast<elem_t<DT>*>(a.poolT) + (((size_t)page * a.rank) << m.page_shift) + (size_t)(pos & ((1 << m.page_shift) - 1)) : nullptr;
   for (int c = lane; c < a.rank; c += 64) {
@@ -230,7 +235,7 @@ __global__ __launch_bounds__(256) void latent_attn_kernel(StepMeta m, LatentAttn
   __shared__ float s_m[4], s_l[4];
   extern __shared__ float s_acc[];      // [4][rank]
   const int t = blockIdx.x, h = blockIdx.y, lane = threadIdx.x & 63, wv = threadIdx.x >> 6;
-  const int row = m.ent_row[m.tok_ent[t]], nkeys = m.tok_pos[t] + 1;
+  const int row = m.tok_row[t], nkeys = m.tok_pos[t] + 1;
   int k0 = 0, k1 = nkeys;
   if (SPLIT) { k0 = min(nkeys, (int)blockIdx.z * a.keys_per); k1 = min(nkeys, k0 + a.keys_per); }
   const float* q = a.q + (size_t)t * a.ldq + (size_t)h * a.rank;
@@ -414,9 +419,9 @@ __global__ void stack_gather_tok_kernel(int* tok_id, const int* ent_row, const i
   const int i = blockIdx.x * blockDim.x + threadIdx.x;
   if (i < S) tok_id[i] = slab_tok[ent_row[i]];
 }
-__global__ void stack_advance_kernel(int* tok_pos, int* ent_par, int S) {
+__global__ void stack_advance_kernel(int* tok_pos, int* ent_par, int* tok_par, int S) {      // one token per entry: token i is entry i
   const int i = blockIdx.x * blockDim.x + threadIdx.x;
-  if (i < S) { tok_pos[i] += 1; ent_par[i] ^= 1; }
+  if (i < S) { tok_pos[i] += 1; ent_par[i] ^= 1; tok_par[i] ^= 1; }
 }
 
 }  // namespace tgx

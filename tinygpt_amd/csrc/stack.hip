@@ -39,18 +39,18 @@ int upload_f32(tgx_ctx* c, float* dst, const void* host, int64_t n, int src_dtyp
 }
 size_t esize(int src_dtype) { return src_dtype == TGX_F32 ? 4 : 2; }
 
-struct MetaPtrs { int *tok_id, *tok_pos, *tok_ent, *ent_row, *ent_start, *ent_count, *ent_par, *want, *want_row; size_t n; };
+struct MetaPtrs { int *tok_id, *tok_pos, *tok_ent, *tok_row, *tok_idx, *tok_cnt, *tok_par, *ent_row, *ent_start, *ent_count, *ent_par, *want, *want_row; size_t n; };
 MetaPtrs meta_layout(int* base, int T, int S, int NW) {
   MetaPtrs p;
-  p.tok_id = base; p.tok_pos = p.tok_id + T; p.tok_ent = p.tok_pos + T;
-  p.ent_row = p.tok_ent + T; p.ent_start = p.ent_row + S; p.ent_count = p.ent_start + S; p.ent_par = p.ent_count + S;
+  p.tok_id = base; p.tok_pos = p.tok_id + T; p.tok_ent = p.tok_pos + T; p.tok_row = p.tok_ent + T; p.tok_idx = p.tok_row + T; p.tok_cnt = p.tok_idx + T; p.tok_par = p.tok_cnt + T;
+  p.ent_row = p.tok_par + T; p.ent_start = p.ent_row + S; p.ent_count = p.ent_start + S; p.ent_par = p.ent_count + S;
   p.want = p.ent_par + S; p.want_row = p.want + NW;
-  p.n = (size_t)3 * T + (size_t)4 * S + (size_t)2 * NW;
+  p.n = (size_t)7 * T + (size_t)4 * S + (size_t)2 * NW;
   return p;
 }
 tgx::StepMeta step_meta(const StackModel* sm, const MetaPtrs& p, int T, int S) {
   tgx::StepMeta m{};
-  m.tok_id = p.tok_id; m.tok_pos = p.tok_pos; m.tok_ent = p.tok_ent; m.ent_row = p.ent_row; m.ent_start = p.ent_start; m.ent_count = p.ent_count; m.ent_par = p.ent_par;
+  m.tok_id = p.tok_id; m.tok_pos = p.tok_pos; m.tok_ent = p.tok_ent; m.tok_row = p.tok_row; m.tok_idx = p.tok_idx; m.tok_cnt = p.tok_cnt; m.tok_par = p.tok_par; m.ent_row = p.ent_row; m.ent_start = p.ent_start; m.ent_count = p.ent_count; m.ent_par = p.ent_par;
   m.tbl = sm->tbl_dev; m.tbl_stride = sm->tbl_stride; m.page_shift = sm->page_shift; m.T = T; m.S = S;
   return m;
 }
@@ -179,7 +179,7 @@ int ensure_ws(tgx_ctx* c, int T) {
         (rc = dev_alloc(c, &sm->tile_e, std::max<size_t>(np / 64, GROUPED_FEW_PAIRS / GROUPED_FEW_ROWS) + (size_t)sm->max_E + 1)) ||
         (rc = dev_alloc(c, &sm->tile_m0, std::max<size_t>(np / 64, GROUPED_FEW_PAIRS / GROUPED_FEW_ROWS) + (size_t)sm->max_E + 1))) return rc;
   }
-  sm->meta_cap = (size_t)5 * n + (size_t)4 * sm->d.max_seqs;
+  sm->meta_cap = (size_t)9 * n + (size_t)4 * sm->d.max_seqs;
   if ((rc = dev_alloc(c, &sm->meta_dev, sm->meta_cap))) return rc;
   HIP_OK(c, hipHostMalloc((void**)&sm->meta_host, sm->meta_cap * 4, hipHostMallocDefault));
   sm->cap_tokens = cap;
@@ -646,7 +646,10 @@ int stack_step(tgx_ctx* c, int S, const int32_t* rows, const int32_t* counts, co
     const int r = rows[e];
     assign_pages(sm, r, c->row_past[(size_t)r] + counts[e]);
     hp.ent_row[e] = r; hp.ent_start[e] = t; hp.ent_count[e] = counts[e]; hp.ent_par[e] = sm->row_par[(size_t)r];
-    for (int i = 0; i < counts[e]; i++, t++) { hp.tok_id[t] = (int)ids[t]; hp.tok_pos[t] = (int)c->row_past[(size_t)r] + i; hp.tok_ent[t] = e; }
+    for (int i = 0; i < counts[e]; i++, t++) {
+      hp.tok_id[t] = (int)ids[t]; hp.tok_pos[t] = (int)c->row_past[(size_t)r] + i; hp.tok_ent[t] = e;
+      hp.tok_row[t] = r; hp.tok_idx[t] = i; hp.tok_cnt[t] = counts[e]; hp.tok_par[t] = sm->row_par[(size_t)r];
+    }
   }
   for (int i = 0; i < n_want; i++) {
     hp.want[i] = want[i]; hp.want_row[i] = 0;
@@ -715,6 +718,7 @@ int stack_decode(tgx_ctx* c, const tgx_sampler_cfg& cfg, uint64_t seed, int n) {
     assign_pages(sm, r, c->row_past[(size_t)r] + n);
     hp.ent_row[e] = r; hp.ent_start[e] = e; hp.ent_count[e] = 1; hp.ent_par[e] = sm->row_par[(size_t)r];
     hp.tok_id[e] = 0; hp.tok_pos[e] = (int)c->row_past[(size_t)r]; hp.tok_ent[e] = e; hp.want[e] = e; hp.want_row[e] = r;
+    hp.tok_row[e] = r; hp.tok_idx[e] = 0; hp.tok_cnt[e] = 1; hp.tok_par[e] = sm->row_par[(size_t)r];
   }
   if ((rc = push_tables(c)) || (rc = push_meta(c, hp.n))) return rc;
   for (int b = 0; b < c->batch; b++) { c->row_probs_cfg[(size_t)b] = cfg; c->row_probs_ok[(size_t)b] = is_greedy(&cfg) ? 0 : 1; }
@@ -725,7 +729,7 @@ int stack_decode(tgx_ctx* c, const tgx_sampler_cfg& cfg, uint64_t seed, int n) {
     run_logits(c, dp.want, S, c->slab_logits, dp.want_row);
     for (int r : live) launch_argmax_partials(c, c->rows[(size_t)r].logits, d.vocab, c->rows[(size_t)r].part_val, c->rows[(size_t)r].part_idx);
     launch_sample(c, 0, c->batch, cfg, /*advance_pos=*/true, /*log_step=*/true);
-    hipLaunchKernelGGL(tgx::stack_advance_kernel, dim3((S + 63) / 64), dim3(64), 0, c->stream, dp.tok_pos, dp.ent_par, S);
+    hipLaunchKernelGGL(tgx::stack_advance_kernel, dim3((S + 63) / 64), dim3(64), 0, c->stream, dp.tok_pos, dp.ent_par, dp.tok_par, S);
     c->steps_issued++;
   }
   HIP_OK(c, hipGetLastError());
