@@ -4,8 +4,8 @@
 //   norm_conv_kernel        grouped RMS norm, the sublayer's causal short convolution over the normed rows, and the slot's convolution state
 //   latent_append_kernel    RMS norm of the down-projected latent and its store into the paged pool
 //   latent_attn_kernel      queries (already multiplied into latent space) against the pool: softmax with a sink, output in latent space
-//   latent_attn_split_kernel / latent_attn_merge_kernel   the same with a sequence's keys divided between workgroups (few tokens, long contexts)
-//   router_topk_kernel      32-bit router logits, top-k, softmax over the chosen
+//   latent_attn_kernel<.., SPLIT> + latent_attn_merge_kernel   the same with a sequence's keys divided between workgroups (few tokens, long contexts)
+//   router_topk_kernel      bias, top-k and softmax over the chosen on the router's fp32 products (stack_gemm.h)
 //   moe_plan_kernel         (token, choice) pairs grouped by expert: offsets, permutation, tile list of the grouped products
 //   combine_depth_kernel    residual + weighted expert outputs, then the learned average over the embedding output and all layer results
 //   final_norm_rows_kernel  grouped RMS norm of the rows whose logits are asked for
