@@ -59,6 +59,7 @@ MECH = {
     "five_taps": dict(canon_taps=5, layers=[plain_layer(), plain_layer()]),
     "one_head": dict(layers=[plain_layer(heads=1, dim=16, vdim=12, kv_rank=24)]),
     "wide_latent": dict(layers=[plain_layer(heads=4, dim=8, vdim=8, kv_rank=160)]),          # several latent channels per lane
+    "very_wide_latent": dict(layers=[plain_layer(heads=2, dim=8, vdim=8, kv_rank=1100)]),
     "sharp_scores": dict(layers=[plain_layer(scale=3.0), plain_layer(scale=3.0)]),            # peaked softmax: single keys carry the output
     "top_one": dict(layers=[moe_layer(top=1)]),
     "top_all": dict(layers=[moe_layer(experts=4, top=4)]),

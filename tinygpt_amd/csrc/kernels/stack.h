@@ -195,7 +195,7 @@ __global__ __launch_bounds__(64) void latent_append_kernel(StepMeta m, LatentApp
 // ---- latent attention, one workgroup per (token, head): the four waves take every fourth key, lanes hold rank / 64 latent channels each.
 // Scores are fp32 dot products of the latent-space query (score scale folded in) with the cached latents; the softmax denominator also holds
 // exp(sink[head]) — a term without key or value that counts once.  The output stays in latent space (the value up-projection follows as a product).
-constexpr int LAT_MAX_RPL = 16;       // latent channels per lane: rank <= 1024
+constexpr int LAT_MAX_RPL = 32;       // latent channels per lane: rank <= 2048
 struct LatentAttnArgs {
   const float* q; long long ldq;      // [T][heads * rank]
   const void* pool;

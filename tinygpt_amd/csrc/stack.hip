@@ -140,7 +140,8 @@ void launch_attn_t(tgx_ctx* c, const tgx::StepMeta& m, const tgx::LatentAttnArgs
   else if (rpl <= 2) hipLaunchKernelGGL((tgx::latent_attn_kernel<DT, 2, SPLIT>), grid, dim3(256), lds, c->stream, m, a);
   else if (rpl <= 4) hipLaunchKernelGGL((tgx::latent_attn_kernel<DT, 4, SPLIT>), grid, dim3(256), lds, c->stream, m, a);
   else if (rpl <= 8) hipLaunchKernelGGL((tgx::latent_attn_kernel<DT, 8, SPLIT>), grid, dim3(256), lds, c->stream, m, a);
-  else hipLaunchKernelGGL((tgx::latent_attn_kernel<DT, 16, SPLIT>), grid, dim3(256), lds, c->stream, m, a);
+  else if (rpl <= 16) hipLaunchKernelGGL((tgx::latent_attn_kernel<DT, 16, SPLIT>), grid, dim3(256), lds, c->stream, m, a);
+  else hipLaunchKernelGGL((tgx::latent_attn_kernel<DT, 32, SPLIT>), grid, dim3(256), lds, c->stream, m, a);
 }
 
 // the matrix-core attention serves 16-bit storage, latent widths of 128 .. 512 in steps of 128, pages of a multiple of 32 tokens
