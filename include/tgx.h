@@ -27,7 +27,7 @@ extern "C" {
 
 /* 3 (round 5): per-row sequence lifecycle (tgx_reset_row / tgx_forward_row / tgx_sample_row / tgx_past_length_row); tgx_get_option added and
  * tgx_engine_read_stats + the options engine.*, pf.*, attn.fold_*, lmhead.fuse_finalize removed since 2. */
-#define TGX_ABI_VERSION 4   /* 4: layered models (tgx_create_stack, tgx_step_ragged) */
+#define TGX_ABI_VERSION 5   /* 4: layered models (tgx_create_stack, tgx_step_ragged); 5: Modepel (more mixers / feed-forward kinds in tgx_layer_desc) */
 
 #if defined(__GNUC__)
 #define TGX_API __attribute__((visibility("default")))
@@ -56,7 +56,8 @@ typedef enum tgx_family {
   TGX_FAMILY_QWEN2 = 3,
   TGX_FAMILY_QWEN3 = 4,
   TGX_FAMILY_MISTRAL = 5,
-  TGX_FAMILY_ZAKUSUN = 6   /* a layered model (tgx_stack_desc below), no counterpart in the reference */
+  TGX_FAMILY_ZAKUSUN = 6,  /* a layered model (tgx_stack_desc below), no counterpart in the reference */
+  TGX_FAMILY_MODEPEL = 7   /* a layered model: rotary grouped-query attention and matrix-memory (mLSTM) layers, sandwich norms */
 } tgx_family;
 
 /* tinytorch::DType values the CLI accepts (examples/inference/main.cpp:82-88) */
@@ -104,9 +105,21 @@ typedef struct tgx_model_desc {
  *                             sink in the denominator, sigmoid output gate
  *   mixture of experts        top-k of a 32-bit router (+ bias), weights = softmax over the chosen logits, clamped gated experts
  *   depth average             the stream handed to layer i + 1 is a learned weighting of the embedding output and all layer results so far
- *   sinusoidal positions      added to the embedding rows (interleaved sin / cos, base 10000) */
-typedef enum tgx_mixer { TGX_MIXER_LATENT_ATTENTION = 1 } tgx_mixer;
-typedef enum tgx_mlp { TGX_MLP_NONE = 0, TGX_MLP_MOE = 1 } tgx_mlp;
+ *   sinusoidal positions      added to the embedding rows (interleaved sin / cos, base 10000)
+ * and, for TGX_FAMILY_MODEPEL (whose slots hold pages of a key / value pool and one recurrent state per mLSTM layer):
+ *   scalar RMS norm           x / sqrt(mean(x^2) + norm_eps) times ONE learned number, before and after every sublayer ("sandwich"):
+ *                             x <- x + norm_b(sublayer(norm_a(x)))
+ *   grouped-query attention   heads query heads over kv_heads cached key / value heads, biases on q / k / v, rotary positions on the first rot_dims
+ *                             dimensions of every head (rotate-half pairing, base rot_base), score scale `scale`, a sink of score 0 without a value
+ *                             in the softmax denominator, values mixed with the first such layer's values of the same token (v_mix), sigmoid output gate
+ *   mLSTM                     matrix memory per head with exponential input gate, sigmoid forget gate (both soft-capped by gate_cap), a running
+ *                             maximum that starts at 0, fp32 state per slot; per-head RMS norm, learned scale, sigmoid output gate
+ *   dense feed-forward        down(PolyNorm(up(h))): a N(z) + b N(z^2) + c N(z^3) + e over a token's ff values
+ *   grouped-choice experts    softmax router over experts + identity outputs; the choice adds a correction and is limited to the best groups_keep of
+ *                             `groups` neighbour groups; weights = scores * router_scale; identity outputs hand the input through; gated-silu
+ *                             experts; a shared expert of width shared_ff with a per-token sigmoid gate */
+typedef enum tgx_mixer { TGX_MIXER_LATENT_ATTENTION = 1, TGX_MIXER_ATTENTION = 2, TGX_MIXER_MLSTM = 3 } tgx_mixer;
+typedef enum tgx_mlp { TGX_MLP_NONE = 0, TGX_MLP_MOE = 1, TGX_MLP_DENSE = 2 } tgx_mlp;
 
 typedef struct tgx_layer_desc {
   int32_t mixer;     /* tgx_mixer                                                                 */
@@ -120,10 +133,21 @@ typedef struct tgx_layer_desc {
   int32_t top;       /* experts per token                                                         */
   int32_t ff;        /* expert width                                                              */
   float limit;       /* clamp of the expert's gate (from above) and up (both sides) projections   */
+  /* ABI 5 (zero for the mixers / feed-forward kinds that do not read them) */
+  int32_t kv_heads;  /* attention: key / value heads (query head h reads head h / (heads / kv_heads)) */
+  int32_t rot_dims;  /* attention: rotated dimensions per head (even, <= dim; 0: none)            */
+  float rot_base;    /* attention: dimension pair i turns by position * rot_base^(-2i / rot_dims) */
+  int32_t v_mix;     /* attention: 1 = values are mixed with the first such layer's values        */
+  float gate_cap;    /* mLSTM: soft cap of the gate pre-activations, cap * tanh(z / cap)          */
+  int32_t identity;  /* experts: router outputs beyond `experts` that hand the input through      */
+  int32_t groups;    /* experts: neighbour groups of router outputs (<= 1: no group limit)        */
+  int32_t groups_keep; /* experts: groups whose members may be chosen                             */
+  float router_scale;  /* experts: weights = scores * router_scale                                */
+  int32_t shared_ff; /* experts: width of the shared expert (0: none)                             */
 } tgx_layer_desc;
 
 typedef struct tgx_stack_desc {
-  int32_t family;         /* tgx_family (TGX_FAMILY_ZAKUSUN)                                       */
+  int32_t family;         /* tgx_family (TGX_FAMILY_ZAKUSUN, TGX_FAMILY_MODEPEL)                   */
   int32_t width;          /* residual width                                                        */
   int32_t layers;         /* entries of the tgx_layer_desc array                                   */
   int32_t vocab;
@@ -158,7 +182,9 @@ TGX_API int tgx_device_count(int* out_count);
 TGX_API int tgx_create(const tgx_model_desc* desc, int device_ordinal, tgx_ctx** out_ctx);
 
 /* The layered counterpart of tgx_create: `layers` holds desc->layers entries.  Checkpoint names (tgx_upload): "embed", "final.norm",
- * "l<i>.norm1|norm2|canon1|canon2|dwa", "l<i>.mix.q|dkv|dkv.norm|uk|uv|sink|g|o", "l<i>.mlp.router|router.b", "l<i>.mlp.e<j>.gate|up|down". */
+ * "l<i>.norm1|norm2|canon1|canon2|dwa", "l<i>.mix.q|dkv|dkv.norm|uk|uv|sink|g|o", "l<i>.mlp.router|router.b", "l<i>.mlp.e<j>.gate|up|down".
+ * TGX_FAMILY_MODEPEL: "embed", "head", "final.norm", "l<i>.norm1|norm1b|norm2|norm2b", attention "l<i>.mix.q|k|v(.b)|vmix|g|o", mLSTM
+ * "l<i>.mix.q|k|v|g|o|norm|i(.b)|f(.b)", dense "l<i>.mlp.up|down|act", experts "l<i>.mlp.router|correction|e<j>.gate|up|down|shared.gate|up|down|sg". */
 TGX_API int tgx_create_stack(const tgx_stack_desc* desc, const tgx_layer_desc* layers, int device_ordinal, tgx_ctx** out_ctx);
 
 /* == SafeTensors::loadInternal -> Storage::copyOnDevice for ONE named tensor

@@ -332,6 +332,7 @@ __global__ __launch_bounds__(64) void router_topk_kernel(RouterArgs a) {
 struct MoePlanArgs {
   const int* sel; int n_pairs, E, top, tile_m;
   int *off, *perm, *tok, *tile_e, *tile_m0, *n_tiles;
+  int E_tiles;               // tiles are made for the first E_tiles experts (0: all); the others' pairs need no product (identity outputs)
 };
 __global__ __launch_bounds__(1024) void moe_plan_kernel(MoePlanArgs a) {
   __shared__ int s_cnt[ROUTER_MAX_E], s_off[ROUTER_MAX_E + 1], s_cur[ROUTER_MAX_E];
@@ -343,7 +344,8 @@ __global__ __launch_bounds__(1024) void moe_plan_kernel(MoePlanArgs a) {
     int o = 0, nt = 0;
     for (int e = 0; e < a.E; e++) {
       s_off[e] = o; a.off[e] = o;
-      for (int m0 = 0; m0 < s_cnt[e]; m0 += a.tile_m) { a.tile_e[nt] = e; a.tile_m0[nt] = o + m0; nt++; }
+      if (a.E_tiles <= 0 || e < a.E_tiles)
+        for (int m0 = 0; m0 < s_cnt[e]; m0 += a.tile_m) { a.tile_e[nt] = e; a.tile_m0[nt] = o + m0; nt++; }
       o += s_cnt[e];
     }
     s_off[a.E] = o; a.off[a.E] = o;

@@ -14,7 +14,8 @@
 
 namespace tgx {
 
-enum { SG_STORE = 0, SG_ADD = 1, SG_GATE = 2, SG_EXPERT_ACT = 3, SG_ROWSCALE = 4 };
+enum { SG_STORE = 0, SG_ADD = 1, SG_GATE = 2, SG_EXPERT_ACT = 3, SG_ROWSCALE = 4, SG_SILU_MUL = 5 };
+constexpr bool sg_dual(int epi) { return epi == SG_EXPERT_ACT || epi == SG_SILU_MUL; }
 struct StackGemmArgs {
   const float* A; long long lda; int a_zoff;
   const int* a_rows;
@@ -23,7 +24,8 @@ struct StackGemmArgs {
   const int* c_rows;
   const int* z_off; const int* tile_z; const int* tile_m0; const int* n_tiles;      // grouped
   int M, N, K;
-  float scale;                 // SG_STORE: C = acc * scale
+  float scale;                 // SG_STORE: C = acc * scale + bias
+  const float* bias;           // SG_STORE: [N] per z (column z * c_zoff + n), nullptr: none
   float limit;                 // SG_EXPERT_ACT
   const float* G; long long ldg; int g_col0;     // SG_GATE: C = acc * sigmoid(G[row][g_col0 + z * c_zoff + n])
   const float* rw;             // SG_ROWSCALE: C = acc * rw[c row]
@@ -35,6 +37,8 @@ __device__ __forceinline__ float expert_act(float gate, float up, float limit) {
   const float g = fminf(gate, limit), u = fminf(fmaxf(up, -limit), limit);
   return g / (1.0f + expf(-1.702f * g)) * (u + 1.0f);
 }
+// the plain gated expert: silu(gate) * up
+__device__ __forceinline__ float silu_mul(float gate, float up) { return gate / (1.0f + expf(-gate)) * up; }
 
 template <int DT, int EPI, bool DUAL, int WT, bool VEC>
 __global__ __launch_bounds__(256) void stack_gemm_kernel(const StackGemmArgs a) {
@@ -218,10 +222,11 @@ __global__ __launch_bounds__(256) void stack_gemm_kernel(const StackGemmArgs a) 
         const int n = n0 + wn * (32 * WT) + j * 32 + (lane & 31);
         if (n >= a.N) continue;
         const float v = acc[0][i][j][r];
-        if constexpr (EPI == SG_STORE) cp[n] = v * a.scale;
+        if constexpr (EPI == SG_STORE) cp[n] = a.bias ? fmaf(v, a.scale, a.bias[(size_t)z * a.c_zoff + n]) : v * a.scale;
         else if constexpr (EPI == SG_ADD) cp[n] += v;
         else if constexpr (EPI == SG_GATE) cp[n] = v / (1.0f + expf(-a.G[crow * a.ldg + a.g_col0 + (size_t)z * a.c_zoff + n]));
         else if constexpr (EPI == SG_EXPERT_ACT) cp[n] = expert_act(v, acc[NB - 1][i][j][r], a.limit);
+        else if constexpr (EPI == SG_SILU_MUL) cp[n] = silu_mul(v, acc[NB - 1][i][j][r]);
         else cp[n] = v * a.rw[crow];
       }
     }
@@ -315,10 +320,11 @@ __global__ __launch_bounds__(256) void stack_gemv_kernel(const StackGemmArgs a) 
       const int n = n0 + j;
       if (n >= a.N) break;
       const float v = acc[0][j][r];
-      if constexpr (EPI == SG_STORE) cp[n] = v * a.scale;
+      if constexpr (EPI == SG_STORE) cp[n] = a.bias ? fmaf(v, a.scale, a.bias[(size_t)z * a.c_zoff + n]) : v * a.scale;
       else if constexpr (EPI == SG_ADD) cp[n] += v;
       else if constexpr (EPI == SG_GATE) cp[n] = v / (1.0f + expf(-a.G[crow * a.ldg + a.g_col0 + (size_t)z * a.c_zoff + n]));
       else if constexpr (EPI == SG_EXPERT_ACT) cp[n] = expert_act(v, acc[NB - 1][j][r], a.limit);
+      else if constexpr (EPI == SG_SILU_MUL) cp[n] = silu_mul(v, acc[NB - 1][j][r]);
       else cp[n] = v * a.rw[crow];
     }
   }

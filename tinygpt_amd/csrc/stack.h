@@ -1,5 +1,6 @@
-// stack.h — host-side state of a layered model (include/tgx.h tgx_stack_desc): per-layer weights, the paged latent pool with its page tables,
-// the slots' convolution state and the workspace of one ragged step.  Owned by tgx_ctx::stack; the launch code lives in stack.hip.
+// stack.h — host-side state of a layered model (include/tgx.h tgx_stack_desc): per-layer weights, the paged cache pool (latents, or keys and values)
+// with its page tables, the slots' convolution / recurrent state and the workspace of one ragged step.  Owned by tgx_ctx::stack; the launch code
+// lives in stack.hip.
 #pragma once
 #include <set>
 #include <string>
@@ -22,13 +23,35 @@ struct StackLayerW {
   ebyte* pool = nullptr;        // latent cache of this layer: [pages][page_tokens][kv_rank]
   ebyte* poolT = nullptr;       // ... and its transposed copy [pages][kv_rank][page_tokens] for the matrix-core attention (layers that take it)
   float* conv_state = nullptr;  // [2 sublayers][2 buffers][slots][taps - 1][width]
+  // sandwich-norm designs: the four norm numbers of the layer live in StackModel::norm_g at 4 * layer (norm1, norm1b, norm2, norm2b)
+  // grouped-query attention: w_in = [q | k | v | gate] rows, bias b_in over the same rows; mLSTM: w_in = [q | k | v | gate | zi | zf]
+  float* b_in = nullptr;        // fp32 [rows of w_in]
+  ebyte* poolV = nullptr;       // attention: values [pages][page_tokens][kv_heads * vdim] (`pool` holds the keys [..][kv_heads * dim])
+  float* vmix = nullptr;        // attention: the value-mixing number
+  int vmode = 0;                // 0: no value mixing, 1: the first mixing layer (its values are handed on), 2: mixes
+  int rot = -1;                 // index of the layer's rotation table (StackModel::rot)
+  float* head_w = nullptr;      // mLSTM: [heads * vdim] scale after the per-head norm
+  float *mS = nullptr, *mn = nullptr, *mm = nullptr;      // mLSTM state: [slots][heads][dim][vdim], [2][slots][heads][dim], [2][slots][heads]
+  // dense feed-forward: w_up [ff][width], w_down [width][ff] (the expert fields), act = PolyNorm's four numbers
+  float* act = nullptr;
+  // grouped-choice experts: w_router holds experts + identity rows and, with a shared expert, its gate row last; b_router is the correction
+  ebyte *ws_gate = nullptr, *ws_up = nullptr, *ws_down = nullptr;      // shared expert
 };
+
+struct RotTable { int dims; float base; float* cs; };      // cos / sin of (position, pair) [max_ctx][dims / 2][2], made on the host in double precision
 
 struct StackModel {
   tgx_stack_desc d{};
   std::vector<StackLayerW> L;
   std::set<std::string> missing;       // checkpoint names not uploaded yet
   float *final_norm = nullptr, *freq = nullptr;
+  // what the family fixes (stack_create): the kind of norm and of layer wiring
+  bool sandwich = false;               // scalar RMS norms before and after every sublayer, no convolutions, no depth average, no position vector, a separate head
+  ebyte* head = nullptr;               // [vocab][width] (sandwich designs; the others multiply by the embedding table)
+  float* norm_g = nullptr;             // [4 * layers + 1] norm numbers, the final norm's last
+  std::vector<RotTable> rot;
+  float *a2 = nullptr, *ytmp = nullptr, *ysh = nullptr, *sgw = nullptr, *vfirst = nullptr, *hs = nullptr;      // more step workspace
+  int max_kvv = 0, max_sff = 0;
   // pages
   int page = 64, page_shift = 6, n_pages = 0, tbl_stride = 0;
   int* tbl_dev = nullptr;

@@ -13,6 +13,7 @@
 #include "kernels/stack.h"
 #include "kernels/stack_gemm.h"
 #include "kernels/stack_attn_mfma.h"
+#include "kernels/stack_seq.h"
 
 int upload_param_ext(tgx_ctx* c, ebyte* dst, const void* host, int64_t n, int src_dtype);      // abi.hip
 
@@ -93,7 +94,7 @@ void launch_gemm(tgx_ctx* c, tgx::StackGemmArgs a, int epi, int nz, int grouped_
   const int kq = dt == tgx::DT_F32 ? 4 : 8;
   const bool vec = a.K % kq == 0 && a.ldb % kq == 0 && a.b_zstride % kq == 0 && a.lda % 4 == 0 && a.a_zoff % 4 == 0 && ((uintptr_t)a.A % 16 == 0) && ((uintptr_t)a.B % 16 == 0) &&
                    (!a.B2 || (uintptr_t)a.B2 % 16 == 0);
-  const bool dual = epi == tgx::SG_EXPERT_ACT;
+  const bool dual = tgx::sg_dual(epi);
   // few rows: the weight-streaming kernel (its loads take whole 8-element slices)
   const bool few = sm->gemv && vec && a.K % 8 == 0 && a.ldb % 8 == 0 && a.b_zstride % 8 == 0 && (a.z_off ? grouped_tile == GROUPED_FEW_ROWS : (a.M <= FEW_ROWS_MAX || a.N <= FEW_COLS_ANY_ROWS));
   if (a.z_off && grouped_tile == GROUPED_FEW_ROWS && !few) { c->launch_fault = "grouped product: the plan was made for the few-row kernel, which these operands cannot take"; return; }
@@ -107,6 +108,7 @@ void launch_gemm(tgx_ctx* c, tgx::StackGemmArgs a, int epi, int nz, int grouped_
         case tgx::SG_ADD: launch_gemv_t<DT, tgx::SG_ADD, false>(c, a, grid, mr); break;
         case tgx::SG_GATE: launch_gemv_t<DT, tgx::SG_GATE, false>(c, a, grid, mr); break;
         case tgx::SG_ROWSCALE: launch_gemv_t<DT, tgx::SG_ROWSCALE, false>(c, a, grid, mr); break;
+        case tgx::SG_SILU_MUL: launch_gemv_t<DT, tgx::SG_SILU_MUL, true>(c, a, grid, mr); break;
         default: if (dual) launch_gemv_t<DT, tgx::SG_EXPERT_ACT, true>(c, a, grid, mr); break;
       })
     return;
@@ -128,6 +130,7 @@ void launch_gemm(tgx_ctx* c, tgx::StackGemmArgs a, int epi, int nz, int grouped_
       case tgx::SG_ADD: launch_gemm_t<DT, tgx::SG_ADD, false>(c, a, g1, g2, wt, vec); break;
       case tgx::SG_GATE: launch_gemm_t<DT, tgx::SG_GATE, false>(c, a, g1, g2, wt, vec); break;
       case tgx::SG_ROWSCALE: launch_gemm_t<DT, tgx::SG_ROWSCALE, false>(c, a, g1, g2, wt, vec); break;
+      case tgx::SG_SILU_MUL: launch_gemm_t<DT, tgx::SG_SILU_MUL, true>(c, a, g1, g2, wt, vec); break;
       default: if (dual) launch_gemm_t<DT, tgx::SG_EXPERT_ACT, true>(c, a, g1, g2, wt, vec); break;
     })
 }
@@ -166,17 +169,22 @@ int ensure_ws(tgx_ctx* c, int T) {
   auto fr = [](auto*& p) { if (p) (void)hipFree(p); p = nullptr; };
   fr(sm->x); fr(sm->xs); fr(sm->a); fr(sm->proj); fr(sm->ql); fr(sm->lat); fr(sm->o); fr(sm->selw); fr(sm->yh); fr(sm->yd); fr(sm->xn); fr(sm->lg);
   fr(sm->sel); fr(sm->perm); fr(sm->ptok); fr(sm->tile_e); fr(sm->tile_m0); fr(sm->meta_dev); fr(sm->zr);
+  fr(sm->a2); fr(sm->ytmp); fr(sm->ysh); fr(sm->sgw); fr(sm->vfirst); fr(sm->hs);
   if (sm->meta_host) { (void)hipHostFree(sm->meta_host); sm->meta_host = nullptr; }
   const int cap = std::max(T, 64);
   const size_t W = (size_t)sm->d.width, n = (size_t)cap;
   int rc;
-  if ((rc = dev_alloc(c, &sm->x, n * W)) || (rc = dev_alloc(c, &sm->xs, (size_t)(sm->d.layers + 1) * n * W)) || (rc = dev_alloc(c, &sm->a, n * W)) ||
+  if (sm->sandwich) {      // no layer results are kept; the seams need a second normed stream, a scratch row and the mixers' side buffers
+    if ((rc = dev_alloc(c, &sm->a2, n * W)) || (rc = dev_alloc(c, &sm->ytmp, n * W)) || (rc = dev_alloc(c, &sm->ysh, n * W)) || (rc = dev_alloc(c, &sm->sgw, n)) ||
+        (rc = dev_alloc(c, &sm->vfirst, n * (size_t)std::max(1, sm->max_kvv))) || (rc = dev_alloc(c, &sm->hs, n * (size_t)std::max(1, sm->max_hv)))) return rc;
+  } else if ((rc = dev_alloc(c, &sm->xs, (size_t)(sm->d.layers + 1) * n * W))) return rc;
+  if ((rc = dev_alloc(c, &sm->x, n * W)) || (rc = dev_alloc(c, &sm->a, n * W)) ||
       (rc = dev_alloc(c, &sm->proj, n * (size_t)sm->max_in)) || (rc = dev_alloc(c, &sm->ql, n * (size_t)sm->max_hr)) || (rc = dev_alloc(c, &sm->lat, n * (size_t)sm->max_hr)) ||
       (rc = dev_alloc(c, &sm->o, n * (size_t)sm->max_hv)) || (rc = dev_alloc(c, &sm->xn, n * W)) || (rc = dev_alloc(c, &sm->lg, n * (size_t)sm->d.vocab))) return rc;
   if (sm->max_top > 0) {
     const size_t np = n * (size_t)sm->max_top;
-    if ((rc = dev_alloc(c, &sm->zr, n * (size_t)sm->max_E)) || (rc = dev_alloc(c, &sm->selw, np)) || (rc = dev_alloc(c, &sm->sel, np)) || (rc = dev_alloc(c, &sm->perm, np)) || (rc = dev_alloc(c, &sm->ptok, np)) ||
-        (rc = dev_alloc(c, &sm->yh, np * (size_t)sm->max_ff)) || (rc = dev_alloc(c, &sm->yd, np * W)) ||
+    if ((rc = dev_alloc(c, &sm->zr, n * (size_t)(sm->max_E + 1))) || (rc = dev_alloc(c, &sm->selw, np)) || (rc = dev_alloc(c, &sm->sel, np)) || (rc = dev_alloc(c, &sm->perm, np)) || (rc = dev_alloc(c, &sm->ptok, np)) ||
+        (rc = dev_alloc(c, &sm->yh, np * (size_t)sm->max_ff + n * (size_t)sm->max_sff)) || (rc = dev_alloc(c, &sm->yd, np * W)) ||
         (rc = dev_alloc(c, &sm->tile_e, std::max<size_t>(np / 64, GROUPED_FEW_PAIRS / GROUPED_FEW_ROWS) + (size_t)sm->max_E + 1)) ||
         (rc = dev_alloc(c, &sm->tile_m0, std::max<size_t>(np / 64, GROUPED_FEW_PAIRS / GROUPED_FEW_ROWS) + (size_t)sm->max_E + 1))) return rc;
   }
@@ -200,7 +208,7 @@ int ensure_part(tgx_ctx* c, size_t elems) {
 }
 
 // the layers of one step; meta is on the device.  max_keys: the longest context any token of the step attends (host knowledge; picks the attention form)
-int run_layers(tgx_ctx* c, const MetaPtrs& mp, int T, int S, int max_keys, int max_count) {
+int run_layers_latent(tgx_ctx* c, const MetaPtrs& mp, int T, int S, int max_keys, int max_count) {
   StackModel* sm = c->stack;
   const tgx::StepMeta m = step_meta(sm, mp, T, S);
   const int W = sm->d.width, nslots = sm->d.max_seqs, nb = sm->d.canon_taps - 1;
@@ -313,13 +321,177 @@ int run_layers(tgx_ctx* c, const MetaPtrs& mp, int T, int S, int max_keys, int m
   return TGX_OK;
 }
 
+// ---- sandwich-norm designs (Modepel): per layer  norm -> mixer -> norm, add  and  norm -> feed-forward -> norm, add.  The seam kernel between two sublayers
+// applies the norm behind one, the residual add and the norm in front of the next, so the stream is read and written once per sublayer.
+template <int DT, bool SPLIT>
+void launch_gqa_t(tgx_ctx* c, const tgx::StepMeta& m, const tgx::GqaAttnArgs& a, dim3 grid) {
+  const size_t lds = (size_t)4 * a.vdim * 4;
+  const int rpl = (std::max(a.dim, a.vdim) + 63) / 64;
+  if (rpl <= 1) hipLaunchKernelGGL((tgx::gqa_attn_kernel<DT, 1, SPLIT>), grid, dim3(256), lds, c->stream, m, a);
+  else if (rpl <= 2) hipLaunchKernelGGL((tgx::gqa_attn_kernel<DT, 2, SPLIT>), grid, dim3(256), lds, c->stream, m, a);
+  else hipLaunchKernelGGL((tgx::gqa_attn_kernel<DT, 4, SPLIT>), grid, dim3(256), lds, c->stream, m, a);
+}
+
+int run_attention(tgx_ctx* c, const tgx::StepMeta& m, StackLayerW& w, const float* hin, int T, int max_keys) {
+  StackModel* sm = c->stack;
+  const tgx_layer_desc& ld = w.d;
+  const int W = sm->d.width, H = ld.heads, G = ld.kv_heads, qd = H * ld.dim, kd = G * ld.dim, kvv = G * ld.vdim, vd = H * ld.vdim, nin = qd + kd + kvv + vd;
+  // [q | k | v | gate] = h . w_in^T + b
+  tgx::StackGemmArgs g{};
+  g.A = hin; g.lda = W; g.B = w.w_in; g.ldb = W; g.C = sm->proj; g.ldc = nin; g.M = T; g.N = nin; g.K = W; g.scale = 1.f; g.bias = w.b_in;
+  launch_gemm(c, g, tgx::SG_STORE, 1);
+  tgx::GqaAppendArgs ap{};
+  ap.proj = sm->proj; ap.ldp = nin; ap.heads = H; ap.kv_heads = G; ap.dim = ld.dim; ap.vdim = ld.vdim; ap.rot_dims = ld.rot_dims;
+  ap.cs = w.rot >= 0 ? sm->rot[(size_t)w.rot].cs : nullptr; ap.poolK = w.pool; ap.poolV = w.poolV; ap.vfirst = sm->vfirst; ap.vmode = w.vmode; ap.lam = w.vmix;
+  TGX_DT_SWITCH(c->dt, hipLaunchKernelGGL(tgx::gqa_append_kernel<DT>, dim3(T), dim3(256), 0, c->stream, m, ap))
+  tgx::GqaAttnArgs aa{};
+  aa.q = sm->proj; aa.ldq = nin; aa.poolK = w.pool; aa.poolV = w.poolV; aa.gate = sm->proj + qd + kd + kvv; aa.ldg = nin; aa.out = sm->o; aa.ldo = vd;
+  aa.heads = H; aa.kv_heads = G; aa.dim = ld.dim; aa.vdim = ld.vdim; aa.scale = ld.scale; aa.sink = 0.f; aa.has_sink = 1;
+  int nsplit = 1;
+  if (max_keys >= sm->attn_split_min_keys && (long long)T * H < 2LL * c->num_cus) {      // few (token, head) pairs and a long context: the keys are divided between workgroups
+    nsplit = (int)std::min<long long>(64, (4LL * c->num_cus) / ((long long)T * H));
+    const int per = std::max(256, ((max_keys + nsplit - 1) / nsplit + 63) / 64 * 64);
+    nsplit = (max_keys + per - 1) / per;
+    aa.keys_per = per;
+  }
+  if (nsplit > 1) {
+    int rc = ensure_part(c, (size_t)T * H * nsplit * (size_t)(ld.vdim + 2));
+    if (rc) return rc;
+    aa.part = sm->part; aa.nsplit = nsplit;
+    TGX_DT_SWITCH(c->dt, (launch_gqa_t<DT, true>(c, m, aa, dim3(T, H, nsplit))))
+    hipLaunchKernelGGL(tgx::gqa_attn_merge_kernel, dim3(T, H), dim3(256), 0, c->stream, aa);
+  } else {
+    TGX_DT_SWITCH(c->dt, (launch_gqa_t<DT, false>(c, m, aa, dim3(T, H))))
+  }
+  // y = o . w_o^T
+  g = tgx::StackGemmArgs{};
+  g.A = sm->o; g.lda = vd; g.B = w.w_o; g.ldb = vd; g.C = sm->yd; g.ldc = W; g.M = T; g.N = W; g.K = vd; g.scale = 1.f;
+  launch_gemm(c, g, tgx::SG_STORE, 1);
+  return TGX_OK;
+}
+
+int run_mlstm(tgx_ctx* c, const tgx::StepMeta& m, StackLayerW& w, const float* hin, int T, int S) {
+  StackModel* sm = c->stack;
+  const tgx_layer_desc& ld = w.d;
+  const int W = sm->d.width, H = ld.heads, qd = H * ld.dim, vd = H * ld.vdim, nin = 2 * qd + 2 * vd + 2 * H;
+  // [q | k | v | gate | zi | zf] = h . w_in^T (+ the gate biases)
+  tgx::StackGemmArgs g{};
+  g.A = hin; g.lda = W; g.B = w.w_in; g.ldb = W; g.C = sm->proj; g.ldc = nin; g.M = T; g.N = nin; g.K = W; g.scale = 1.f; g.bias = w.b_in;
+  launch_gemm(c, g, tgx::SG_STORE, 1);
+  tgx::MlstmArgs ma{};
+  ma.proj = sm->proj; ma.ldp = nin; ma.heads = H; ma.dim = ld.dim; ma.vdim = ld.vdim; ma.cap = ld.gate_cap; ma.qscale = 1.0f / sqrtf((float)ld.dim);
+  ma.S = w.mS; ma.n = w.mn; ma.mx = w.mm; ma.n_buf = (size_t)sm->d.max_seqs * H * ld.dim; ma.mx_buf = (size_t)sm->d.max_seqs * H;
+  ma.hs = sm->hs; ma.ldh = vd;
+  const dim3 grid(S, H, (ld.vdim + 63) / 64);
+  const int dper = (ld.dim + 3) / 4;
+  if (dper <= 16) hipLaunchKernelGGL(tgx::mlstm_scan_kernel<16>, grid, dim3(256), 0, c->stream, m, ma);
+  else if (dper <= 32) hipLaunchKernelGGL(tgx::mlstm_scan_kernel<32>, grid, dim3(256), 0, c->stream, m, ma);
+  else if (dper <= 64) hipLaunchKernelGGL(tgx::mlstm_scan_kernel<64>, grid, dim3(256), 0, c->stream, m, ma);
+  else hipLaunchKernelGGL(tgx::mlstm_scan_kernel<128>, grid, dim3(256), 0, c->stream, m, ma);
+  tgx::MlstmOutArgs oa{};
+  oa.hs = sm->hs; oa.ldh = vd; oa.w = w.head_w; oa.gate = sm->proj + 2 * qd + vd; oa.ldg = nin; oa.out = sm->o; oa.ldo = vd; oa.vdim = ld.vdim; oa.eps = sm->d.norm_eps;
+  hipLaunchKernelGGL(tgx::mlstm_out_kernel, dim3(T, H), dim3(64), 0, c->stream, oa);
+  g = tgx::StackGemmArgs{};
+  g.A = sm->o; g.lda = vd; g.B = w.w_o; g.ldb = vd; g.C = sm->yd; g.ldc = W; g.M = T; g.N = W; g.K = vd; g.scale = 1.f;
+  launch_gemm(c, g, tgx::SG_STORE, 1);
+  return TGX_OK;
+}
+
+void run_dense_ff(tgx_ctx* c, StackLayerW& w, const float* hin, int T) {
+  StackModel* sm = c->stack;
+  const int W = sm->d.width, F = w.d.ff;
+  tgx::StackGemmArgs g{};
+  g.A = hin; g.lda = W; g.B = w.w_up; g.ldb = W; g.C = sm->yh; g.ldc = F; g.M = T; g.N = F; g.K = W; g.scale = 1.f;
+  launch_gemm(c, g, tgx::SG_STORE, 1);
+  hipLaunchKernelGGL(tgx::poly_norm_kernel, dim3(T), dim3(256), 0, c->stream, sm->yh, w.act, F, sm->d.norm_eps);
+  g = tgx::StackGemmArgs{};
+  g.A = sm->yh; g.lda = F; g.B = w.w_down; g.ldb = F; g.C = sm->yd; g.ldc = W; g.M = T; g.N = W; g.K = F; g.scale = 1.f;
+  launch_gemm(c, g, tgx::SG_STORE, 1);
+}
+
+// grouped-choice experts: the chosen pairs' rows land in yd (none for identity outputs), the shared expert's in ysh; the seam kernel sums them
+void run_choice_experts(tgx_ctx* c, StackLayerW& w, const float* hin, int T) {
+  StackModel* sm = c->stack;
+  const tgx_layer_desc& ld = w.d;
+  const int W = sm->d.width, E = ld.experts + ld.identity, top = ld.top, nz = E + (ld.shared_ff > 0 ? 1 : 0);
+  tgx::StackGemmArgs g{};
+  g.A = hin; g.lda = W; g.B = w.w_router; g.ldb = W; g.C = sm->zr; g.ldc = nz; g.M = T; g.N = nz; g.K = W; g.scale = 1.f;
+  launch_gemm(c, g, tgx::SG_STORE, 1, 0, 0, 64, tgx::DT_F32);
+  tgx::RouterGroupArgs ra{};
+  ra.z = sm->zr; ra.ldz = nz; ra.corr = w.b_router; ra.sel = sm->sel; ra.selw = sm->selw; ra.sgw = ld.shared_ff > 0 ? sm->sgw : nullptr;
+  ra.E = E; ra.top = top; ra.groups = ld.groups; ra.keep = ld.groups_keep; ra.scale = ld.router_scale;
+  hipLaunchKernelGGL(tgx::router_group_kernel, dim3(T), dim3(64), 0, c->stream, ra);
+  const int np = T * top;
+  if (ld.experts > 0) {
+    tgx::MoePlanArgs pa{};
+    pa.sel = sm->sel; pa.n_pairs = np; pa.E = E; pa.top = top; pa.tile_m = grouped_tile_rows(c, np, W, ld.ff); pa.E_tiles = ld.experts;
+    pa.off = sm->moe_off; pa.perm = sm->perm; pa.tok = sm->ptok; pa.tile_e = sm->tile_e; pa.tile_m0 = sm->tile_m0; pa.n_tiles = sm->n_tiles;
+    hipLaunchKernelGGL(tgx::moe_plan_kernel, dim3(1), dim3(1024), 0, c->stream, pa);
+    g = tgx::StackGemmArgs{};
+    g.A = hin; g.lda = W; g.a_rows = sm->ptok; g.B = w.w_gate; g.B2 = w.w_up; g.ldb = W; g.b_zstride = (long long)ld.ff * W; g.C = sm->yh; g.ldc = ld.ff;
+    g.z_off = sm->moe_off; g.tile_z = sm->tile_e; g.tile_m0 = sm->tile_m0; g.n_tiles = sm->n_tiles; g.M = np; g.N = ld.ff; g.K = W;
+    launch_gemm(c, g, tgx::SG_SILU_MUL, 1, np, E, pa.tile_m);
+    g = tgx::StackGemmArgs{};
+    g.A = sm->yh; g.lda = ld.ff; g.B = w.w_down; g.ldb = ld.ff; g.b_zstride = (long long)W * ld.ff; g.C = sm->yd; g.ldc = W; g.c_rows = sm->perm;
+    g.z_off = sm->moe_off; g.tile_z = sm->tile_e; g.tile_m0 = sm->tile_m0; g.n_tiles = sm->n_tiles; g.M = np; g.N = W; g.K = ld.ff; g.rw = sm->selw;
+    launch_gemm(c, g, tgx::SG_ROWSCALE, 1, np, E, pa.tile_m);
+  }
+  if (ld.shared_ff > 0) {
+    float* hsh = sm->yh + (size_t)np * std::max(1, ld.ff);
+    g = tgx::StackGemmArgs{};
+    g.A = hin; g.lda = W; g.B = w.ws_gate; g.B2 = w.ws_up; g.ldb = W; g.C = hsh; g.ldc = ld.shared_ff; g.M = T; g.N = ld.shared_ff; g.K = W;
+    launch_gemm(c, g, tgx::SG_SILU_MUL, 1);
+    g = tgx::StackGemmArgs{};
+    g.A = hsh; g.lda = ld.shared_ff; g.B = w.ws_down; g.ldb = ld.shared_ff; g.C = sm->ysh; g.ldc = W; g.M = T; g.N = W; g.K = ld.shared_ff; g.rw = sm->sgw;
+    launch_gemm(c, g, tgx::SG_ROWSCALE, 1);
+  }
+}
+
+int run_layers_sandwich(tgx_ctx* c, const MetaPtrs& mp, int T, int S, int max_keys) {
+  StackModel* sm = c->stack;
+  const tgx::StepMeta m = step_meta(sm, mp, T, S);
+  const int W = sm->d.width, L = sm->d.layers;
+  const float eps = sm->d.norm_eps;
+  TGX_DT_SWITCH(c->dt, hipLaunchKernelGGL(tgx::embed_rows_kernel<DT>, dim3(T), dim3(256), 0, c->stream, m, reinterpret_cast<const tgx::elem_t<DT>*>(c->embed), sm->x, W))
+  hipLaunchKernelGGL(tgx::scalar_norm_kernel, dim3(T), dim3(256), 0, c->stream, sm->x, nullptr, sm->norm_g, sm->a, W, eps);
+  float *hin = sm->a, *hout = sm->a2;
+  for (int li = 0; li < L; li++) {
+    StackLayerW& w = sm->L[(size_t)li];
+    const tgx_layer_desc& ld = w.d;
+    const float* ng = sm->norm_g + 4 * (size_t)li;
+    const float* next_layer = li + 1 < L ? ng + 4 : nullptr;
+    int rc = ld.mixer == TGX_MIXER_ATTENTION ? run_attention(c, m, w, hin, T, max_keys) : run_mlstm(c, m, w, hin, T, S);
+    if (rc) return rc;
+    tgx::SandwichArgs sa{};
+    sa.x = sm->x; sa.y = sm->yd; sa.top = 1; sa.ytmp = sm->ytmp; sa.g_post = ng + 1; sa.g_next = ld.mlp != TGX_MLP_NONE ? ng + 2 : next_layer; sa.out = hout; sa.W = W; sa.eps = eps;
+    hipLaunchKernelGGL(tgx::sandwich_kernel, dim3(T), dim3(256), 0, c->stream, sa);
+    std::swap(hin, hout);
+    if (ld.mlp == TGX_MLP_NONE) continue;
+    sa = tgx::SandwichArgs{};
+    sa.x = sm->x; sa.y = sm->yd; sa.top = 1; sa.ytmp = sm->ytmp; sa.g_post = ng + 3; sa.g_next = next_layer; sa.out = hout; sa.W = W; sa.eps = eps;
+    if (ld.mlp == TGX_MLP_DENSE) run_dense_ff(c, w, hin, T);
+    else {
+      run_choice_experts(c, w, hin, T);
+      sa.top = ld.top; sa.sel = sm->sel; sa.selw = sm->selw; sa.n_real = ld.experts; sa.h = hin; sa.ysh = ld.shared_ff > 0 ? sm->ysh : nullptr;
+    }
+    hipLaunchKernelGGL(tgx::sandwich_kernel, dim3(T), dim3(256), 0, c->stream, sa);
+    std::swap(hin, hout);
+  }
+  return TGX_OK;
+}
+
+int run_layers(tgx_ctx* c, const MetaPtrs& mp, int T, int S, int max_keys, int max_count) {
+  return c->stack->sandwich ? run_layers_sandwich(c, mp, T, S, max_keys) : run_layers_latent(c, mp, T, S, max_keys, max_count);
+}
+
 // logits of the rows listed in want_dev (indices into the step's tokens): C[crow(i)] = embed . norm(x[want[i]]) * logit_scale
 void run_logits(tgx_ctx* c, const int* want_dev, int nw, float* C, const int* c_rows) {
   StackModel* sm = c->stack;
   const int W = sm->d.width, V = sm->d.vocab;
-  hipLaunchKernelGGL(tgx::final_norm_rows_kernel, dim3(nw), dim3(256), 0, c->stream, sm->x, want_dev, sm->final_norm, sm->xn, W, sm->d.norm_groups, sm->d.norm_eps);
+  if (sm->sandwich) hipLaunchKernelGGL(tgx::scalar_norm_kernel, dim3(nw), dim3(256), 0, c->stream, sm->x, want_dev, sm->norm_g + 4 * (size_t)sm->d.layers, sm->xn, W, sm->d.norm_eps);
+  else hipLaunchKernelGGL(tgx::final_norm_rows_kernel, dim3(nw), dim3(256), 0, c->stream, sm->x, want_dev, sm->final_norm, sm->xn, W, sm->d.norm_groups, sm->d.norm_eps);
   tgx::StackGemmArgs g{};
-  g.A = sm->xn; g.lda = W; g.B = c->embed; g.ldb = W; g.C = C; g.ldc = V; g.c_rows = c_rows; g.M = nw; g.N = V; g.K = W; g.scale = sm->d.logit_scale;
+  g.A = sm->xn; g.lda = W; g.B = sm->head ? sm->head : c->embed; g.ldb = W; g.C = C; g.ldc = V; g.c_rows = c_rows; g.M = nw; g.N = V; g.K = W; g.scale = sm->d.logit_scale;
   launch_gemm(c, g, tgx::SG_STORE, 1);
 }
 
@@ -365,6 +537,162 @@ void refresh_rows(tgx_ctx* c) {
   c->past = m; c->have_token = live > 0 && all;
 }
 
+// parameter storage of a sandwich-norm design (Modepel): per layer the four norm numbers, the mixer's merged input projection with its bias row, the
+// output projection, and the feed-forward of its kind
+int create_sandwich_layers(tgx_ctx* c, const tgx_layer_desc* layers) {
+  StackModel* sm = c->stack;
+  const tgx_stack_desc& d = sm->d;
+  const size_t W = (size_t)d.width, es = c->esz;
+  int rc;
+  if ((rc = dev_alloc(c, &sm->head, (size_t)d.vocab * W * es)) || (rc = dev_alloc(c, &sm->norm_g, (size_t)4 * d.layers + 1))) return rc;
+  HIP_OK(c, hipMemset(sm->norm_g, 0, ((size_t)4 * d.layers + 1) * 4));
+  sm->missing.insert("head");
+  sm->max_top = 1; sm->max_E = 1; sm->max_ff = 1;      // the mixers' outputs and the dense feed-forward use the expert buffers with one row per token
+  bool mixing = false;
+  for (int i = 0; i < d.layers; i++) {
+    StackLayerW& w = sm->L[(size_t)i];
+    w.d = layers[i];
+    const tgx_layer_desc& l = w.d;
+    const std::string p = "l" + std::to_string(i) + ".";
+    const size_t H = (size_t)l.heads, qd = H * l.dim, vd = H * l.vdim;
+    size_t nin;
+    for (const char* n : {"norm1", "norm1b", "mix.q", "mix.k", "mix.v", "mix.g", "mix.o"}) sm->missing.insert(p + n);
+    if (l.mixer == TGX_MIXER_ATTENTION) {
+      const size_t kd = (size_t)l.kv_heads * l.dim, kvv = (size_t)l.kv_heads * l.vdim;
+      nin = qd + kd + kvv + vd;
+      for (const char* n : {"mix.q.b", "mix.k.b", "mix.v.b"}) sm->missing.insert(p + n);
+      if (l.v_mix) {
+        if ((rc = dev_alloc(c, &w.vmix, 1))) return rc;
+        HIP_OK(c, hipMemset(w.vmix, 0, 4));
+        sm->missing.insert(p + "mix.vmix");
+        w.vmode = mixing ? 2 : 1;
+        mixing = true;
+      }
+      if (l.rot_dims > 0) {
+        for (size_t r = 0; r < sm->rot.size(); r++) if (sm->rot[r].dims == l.rot_dims && sm->rot[r].base == l.rot_base) w.rot = (int)r;
+        if (w.rot < 0) { w.rot = (int)sm->rot.size(); sm->rot.push_back(RotTable{l.rot_dims, l.rot_base, nullptr}); }
+      }
+      sm->max_kvv = std::max(sm->max_kvv, (int)kvv);
+    } else {
+      nin = 2 * qd + 2 * vd + 2 * H;
+      if ((rc = dev_alloc(c, &w.head_w, vd))) return rc;
+      for (const char* n : {"mix.norm", "mix.i", "mix.i.b", "mix.f", "mix.f.b"}) sm->missing.insert(p + n);
+    }
+    if ((rc = dev_alloc(c, &w.w_in, nin * W * es)) || (rc = dev_alloc(c, &w.b_in, nin)) || (rc = dev_alloc(c, &w.w_o, W * vd * es))) return rc;
+    HIP_OK(c, hipMemset(w.b_in, 0, nin * 4));
+    sm->max_in = std::max(sm->max_in, (int)nin); sm->max_hv = std::max(sm->max_hv, (int)vd);
+    if (l.mlp == TGX_MLP_NONE) continue;
+    for (const char* n : {"norm2", "norm2b"}) sm->missing.insert(p + n);
+    if (l.mlp == TGX_MLP_DENSE) {
+      const size_t F = (size_t)l.ff;
+      if ((rc = dev_alloc(c, &w.w_up, F * W * es)) || (rc = dev_alloc(c, &w.w_down, W * F * es)) || (rc = dev_alloc(c, &w.act, 4))) return rc;
+      for (const char* n : {"mlp.up", "mlp.down", "mlp.act"}) sm->missing.insert(p + n);
+      sm->max_ff = std::max(sm->max_ff, l.ff);
+      continue;
+    }
+    const size_t E = (size_t)l.experts, Et = E + (size_t)l.identity, F = (size_t)l.ff, SF = (size_t)l.shared_ff;
+    if ((rc = dev_alloc(c, &w.w_router, (Et + 1) * W)) || (rc = dev_alloc(c, &w.b_router, Et))) return rc;
+    for (const char* n : {"mlp.router", "mlp.correction"}) sm->missing.insert(p + n);
+    if (E > 0) {
+      if ((rc = dev_alloc(c, &w.w_gate, E * F * W * es)) || (rc = dev_alloc(c, &w.w_up, E * F * W * es)) || (rc = dev_alloc(c, &w.w_down, E * W * F * es))) return rc;
+      for (int e = 0; e < l.experts; e++)
+        for (const char* n : {".gate", ".up", ".down"}) sm->missing.insert(p + "mlp.e" + std::to_string(e) + n);
+    }
+    if (SF > 0) {
+      if ((rc = dev_alloc(c, &w.ws_gate, SF * W * es)) || (rc = dev_alloc(c, &w.ws_up, SF * W * es)) || (rc = dev_alloc(c, &w.ws_down, W * SF * es))) return rc;
+      for (const char* n : {"mlp.shared.gate", "mlp.shared.up", "mlp.shared.down", "mlp.shared.sg"}) sm->missing.insert(p + n);
+    }
+    sm->max_top = std::max(sm->max_top, l.top); sm->max_ff = std::max(sm->max_ff, l.ff); sm->max_E = std::max(sm->max_E, (int)Et); sm->max_sff = std::max(sm->max_sff, l.shared_ff);
+  }
+  return TGX_OK;
+}
+
+// tensors of a sandwich-norm design by checkpoint name.  A norm is one number (shape [] or [1]).
+int upload_sandwich(tgx_ctx* c, const char* name, const void* host, const int64_t* shape, int nd, int src_dtype) {
+  StackModel* sm = c->stack;
+  const tgx_stack_desc& d = sm->d;
+  const int64_t W = d.width;
+  const bool probe = nd < 0;
+  auto bad_shape = [&]() { return set_err(c, TGX_ERR_SHAPE, "shape not equal for tensor: %s", name); };
+  auto is = [&](int64_t a, int64_t b) { return b < 0 ? (nd == 1 && shape[0] == a) : (nd == 2 && shape[0] == a && shape[1] == b); };
+  auto is_one = [&]() { return nd == 0 || (nd == 1 && shape[0] == 1); };
+  auto done = [&](int rc) { if (!rc) sm->missing.erase(name); return rc; };
+  auto mat = [&](ebyte* dst, int64_t row0, int64_t rows, int64_t cols) {
+    if (probe) return (int)TGX_ERR_SHAPE;
+    if (!is(rows, cols)) return bad_shape();
+    return done(upload_param_ext(c, dst + (size_t)(row0 * cols) * c->esz, host, rows * cols, src_dtype));
+  };
+  auto vec = [&](float* dst, int64_t n) {
+    if (probe) return (int)TGX_ERR_SHAPE;
+    if (!(n == 1 ? is_one() : is(n, -1))) return bad_shape();
+    return done(upload_f32(c, dst, host, n, src_dtype));
+  };
+  if (!strcmp(name, "embed")) return mat(c->embed, 0, d.vocab, W);
+  if (!strcmp(name, "head")) return mat(sm->head, 0, d.vocab, W);
+  if (!strcmp(name, "final.norm")) return vec(sm->norm_g + 4 * (size_t)d.layers, 1);
+  int li = -1;
+  char rest[128] = {0};
+  if (sscanf(name, "l%d.%127s", &li, rest) != 2 || li < 0 || li >= d.layers) return set_err(c, TGX_ERR_NAME, "Unexpected key: %s", name);
+  StackLayerW& w = sm->L[(size_t)li];
+  const tgx_layer_desc& l = w.d;
+  const int64_t H = l.heads, qd = H * l.dim, vd = H * l.vdim;
+  float* ng = sm->norm_g + 4 * (size_t)li;
+  if (!strcmp(rest, "norm1")) return vec(ng, 1);
+  if (!strcmp(rest, "norm1b")) return vec(ng + 1, 1);
+  if (l.mlp != TGX_MLP_NONE && !strcmp(rest, "norm2")) return vec(ng + 2, 1);
+  if (l.mlp != TGX_MLP_NONE && !strcmp(rest, "norm2b")) return vec(ng + 3, 1);
+  if (!strcmp(rest, "mix.o")) return mat(w.w_o, 0, W, vd);
+  if (l.mixer == TGX_MIXER_ATTENTION) {
+    const int64_t kd = (int64_t)l.kv_heads * l.dim, kvv = (int64_t)l.kv_heads * l.vdim;
+    if (!strcmp(rest, "mix.q")) return mat(w.w_in, 0, qd, W);
+    if (!strcmp(rest, "mix.k")) return mat(w.w_in, qd, kd, W);
+    if (!strcmp(rest, "mix.v")) return mat(w.w_in, qd + kd, kvv, W);
+    if (!strcmp(rest, "mix.g")) return mat(w.w_in, qd + kd + kvv, vd, W);
+    if (!strcmp(rest, "mix.q.b")) return vec(w.b_in, qd);
+    if (!strcmp(rest, "mix.k.b")) return vec(w.b_in + qd, kd);
+    if (!strcmp(rest, "mix.v.b")) return vec(w.b_in + qd + kd, kvv);
+    if (w.vmix && !strcmp(rest, "mix.vmix")) return vec(w.vmix, 1);
+  } else {
+    if (!strcmp(rest, "mix.q")) return mat(w.w_in, 0, qd, W);
+    if (!strcmp(rest, "mix.k")) return mat(w.w_in, qd, qd, W);
+    if (!strcmp(rest, "mix.v")) return mat(w.w_in, 2 * qd, vd, W);
+    if (!strcmp(rest, "mix.g")) return mat(w.w_in, 2 * qd + vd, vd, W);
+    if (!strcmp(rest, "mix.i")) return mat(w.w_in, 2 * qd + 2 * vd, H, W);
+    if (!strcmp(rest, "mix.f")) return mat(w.w_in, 2 * qd + 2 * vd + H, H, W);
+    if (!strcmp(rest, "mix.i.b")) return vec(w.b_in + 2 * qd + 2 * vd, H);
+    if (!strcmp(rest, "mix.f.b")) return vec(w.b_in + 2 * qd + 2 * vd + H, H);
+    if (!strcmp(rest, "mix.norm")) return vec(w.head_w, vd);
+  }
+  if (l.mlp == TGX_MLP_DENSE) {
+    if (!strcmp(rest, "mlp.up")) return mat(w.w_up, 0, l.ff, W);
+    if (!strcmp(rest, "mlp.down")) return mat(w.w_down, 0, W, l.ff);
+    if (!strcmp(rest, "mlp.act")) return vec(w.act, 4);
+  }
+  if (l.mlp == TGX_MLP_MOE) {
+    const int64_t E = l.experts, Et = E + l.identity, F = l.ff, SF = l.shared_ff;
+    if (!strcmp(rest, "mlp.router")) { if (probe) return TGX_ERR_SHAPE; if (!is(Et, W)) return bad_shape(); return done(upload_f32(c, w.w_router, host, Et * W, src_dtype)); }
+    if (!strcmp(rest, "mlp.correction")) return vec(w.b_router, Et);
+    if (SF > 0) {
+      if (!strcmp(rest, "mlp.shared.gate")) return mat(w.ws_gate, 0, SF, W);
+      if (!strcmp(rest, "mlp.shared.up")) return mat(w.ws_up, 0, SF, W);
+      if (!strcmp(rest, "mlp.shared.down")) return mat(w.ws_down, 0, W, SF);
+      if (!strcmp(rest, "mlp.shared.sg")) {      // the shared expert's gate row rides behind the router rows: one fp32 product serves both
+        if (probe) return TGX_ERR_SHAPE;
+        if (!is(1, W) && !is(W, -1)) return bad_shape();
+        return done(upload_f32(c, w.w_router + (size_t)(Et * W), host, W, src_dtype));
+      }
+    }
+    int e = -1;
+    char leaf[32] = {0};
+    if (sscanf(rest, "mlp.e%d.%31s", &e, leaf) == 2 && e >= 0 && e < E) {
+      if (!strcmp(leaf, "gate")) return mat(w.w_gate, e * F, F, W);
+      if (!strcmp(leaf, "up")) return mat(w.w_up, e * F, F, W);
+      if (!strcmp(leaf, "down")) return mat(w.w_down, e * W, W, F);
+    }
+  }
+  return set_err(c, TGX_ERR_NAME, "Unexpected key: %s", name);
+}
+
 }  // namespace
 
 // ================================================================================================================================================
@@ -372,15 +700,44 @@ int stack_create(const tgx_stack_desc* desc, const tgx_layer_desc* layers, int d
   if (!desc || !layers || !out_ctx) return set_err(nullptr, TGX_ERR_INVALID, "null argument");
   *out_ctx = nullptr;
   const tgx_stack_desc& d = *desc;
-  if (d.family != TGX_FAMILY_ZAKUSUN) return set_err(nullptr, TGX_ERR_UNSUPPORTED, "family %d is not a layered model", d.family);
+  if (d.family != TGX_FAMILY_ZAKUSUN && d.family != TGX_FAMILY_MODEPEL) return set_err(nullptr, TGX_ERR_UNSUPPORTED, "family %d is not a layered model", d.family);
+  const bool sandwich = d.family == TGX_FAMILY_MODEPEL;
   if (d.width <= 0 || d.layers <= 0 || d.vocab <= 0 || d.max_seqs <= 0 || d.max_ctx <= 0) return set_err(nullptr, TGX_ERR_INVALID, "non-positive model dimension");
   if (d.compute_dtype != TGX_BF16 && d.compute_dtype != TGX_F16 && d.compute_dtype != TGX_F32) return set_err(nullptr, TGX_ERR_INVALID, "unknown compute dtype %d", d.compute_dtype);
-  if (d.norm_groups < 1 || d.norm_groups > tgx::NORM_MAX_GROUPS || d.width % d.norm_groups) return set_err(nullptr, TGX_ERR_UNSUPPORTED, "norm groups %d: 1..%d, dividing the width", d.norm_groups, tgx::NORM_MAX_GROUPS);
-  if (d.canon_taps < 1 || d.canon_taps > tgx::CONV_MAX_TAPS) return set_err(nullptr, TGX_ERR_UNSUPPORTED, "convolution taps %d: 1..%d", d.canon_taps, tgx::CONV_MAX_TAPS);
+  if (!sandwich && (d.norm_groups < 1 || d.norm_groups > tgx::NORM_MAX_GROUPS || d.width % d.norm_groups)) return set_err(nullptr, TGX_ERR_UNSUPPORTED, "norm groups %d: 1..%d, dividing the width", d.norm_groups, tgx::NORM_MAX_GROUPS);
+  if (!sandwich && (d.canon_taps < 1 || d.canon_taps > tgx::CONV_MAX_TAPS)) return set_err(nullptr, TGX_ERR_UNSUPPORTED, "convolution taps %d: 1..%d", d.canon_taps, tgx::CONV_MAX_TAPS);
   int page = d.page_tokens > 0 ? d.page_tokens : 64;
   if (page & (page - 1)) return set_err(nullptr, TGX_ERR_INVALID, "page_tokens %d is not a power of two", page);
+  int first_mix = -1;
   for (int i = 0; i < d.layers; i++) {
     const tgx_layer_desc& l = layers[i];
+    if (sandwich) {
+      if (l.mixer != TGX_MIXER_ATTENTION && l.mixer != TGX_MIXER_MLSTM) return set_err(nullptr, TGX_ERR_UNSUPPORTED, "layer %d: mixer %d is not part of this family (attention and mlstm are)", i, l.mixer);
+      if (l.heads <= 0 || l.dim <= 0 || l.vdim <= 0) return set_err(nullptr, TGX_ERR_INVALID, "layer %d: non-positive mixer size", i);
+      if (l.mixer == TGX_MIXER_ATTENTION) {
+        if (l.kv_heads <= 0 || l.heads % l.kv_heads) return set_err(nullptr, TGX_ERR_INVALID, "layer %d: %d query heads over %d key / value heads", i, l.heads, l.kv_heads);
+        if (l.dim > 64 * tgx::GQA_MAX_RPL || l.vdim > 64 * tgx::GQA_MAX_RPL) return set_err(nullptr, TGX_ERR_UNSUPPORTED, "layer %d: head sizes %d / %d > %d", i, l.dim, l.vdim, 64 * tgx::GQA_MAX_RPL);
+        if (l.rot_dims < 0 || l.rot_dims > l.dim || (l.rot_dims & 1) || (l.rot_dims > 0 && !(l.rot_base > 0.f))) return set_err(nullptr, TGX_ERR_INVALID, "layer %d: %d rotated dimensions of %d (base %g)", i, l.rot_dims, l.dim, l.rot_base);
+        if (l.v_mix) {
+          if (first_mix >= 0 && layers[first_mix].kv_heads * layers[first_mix].vdim != l.kv_heads * l.vdim)
+            return set_err(nullptr, TGX_ERR_INVALID, "layer %d: value mixing needs the value size of layer %d (%d != %d)", i, first_mix, l.kv_heads * l.vdim, layers[first_mix].kv_heads * layers[first_mix].vdim);
+          if (first_mix < 0) first_mix = i;
+        }
+      } else {
+        if (l.dim > 512) return set_err(nullptr, TGX_ERR_UNSUPPORTED, "layer %d: mlstm key size %d > 512", i, l.dim);
+        if (!(l.gate_cap > 0.f)) return set_err(nullptr, TGX_ERR_INVALID, "layer %d: gate_cap %g", i, l.gate_cap);
+      }
+      if (l.mlp != TGX_MLP_NONE && l.mlp != TGX_MLP_MOE && l.mlp != TGX_MLP_DENSE) return set_err(nullptr, TGX_ERR_UNSUPPORTED, "layer %d: feed-forward kind %d is not implemented", i, l.mlp);
+      if (l.mlp == TGX_MLP_DENSE && l.ff <= 0) return set_err(nullptr, TGX_ERR_INVALID, "layer %d: ff %d", i, l.ff);
+      if (l.mlp == TGX_MLP_MOE) {
+        const int E = l.experts + l.identity;
+        if (l.experts < 0 || l.identity < 0 || E <= 0 || E >= tgx::ROUTER_MAX_E || l.top <= 0 || l.top > E || l.top > tgx::ROUTER_MAX_TOP || (l.experts > 0 && l.ff <= 0) || l.shared_ff < 0)
+          return set_err(nullptr, TGX_ERR_UNSUPPORTED, "layer %d: experts %d + identity %d (< %d), top %d (<= %d), ff %d", i, l.experts, l.identity, tgx::ROUTER_MAX_E, l.top, tgx::ROUTER_MAX_TOP, l.ff);
+        if (l.groups > 1 && (E % l.groups || l.groups_keep < 1 || l.groups_keep > l.groups || (long long)l.groups_keep * (E / l.groups) < l.top))
+          return set_err(nullptr, TGX_ERR_INVALID, "layer %d: %d router outputs in %d groups, %d kept, top %d", i, E, l.groups, l.groups_keep, l.top);
+      }
+      continue;
+    }
     if (l.mixer != TGX_MIXER_LATENT_ATTENTION) return set_err(nullptr, TGX_ERR_UNSUPPORTED, "layer %d: mixer %d is not implemented (latent_attention is)", i, l.mixer);
     if (l.heads <= 0 || l.dim <= 0 || l.vdim <= 0 || l.kv_rank <= 0) return set_err(nullptr, TGX_ERR_INVALID, "layer %d: non-positive mixer size", i);
     if (l.kv_rank > 64 * tgx::LAT_MAX_RPL) return set_err(nullptr, TGX_ERR_UNSUPPORTED, "layer %d: kv_rank %d > %d", i, l.kv_rank, 64 * tgx::LAT_MAX_RPL);
@@ -402,7 +759,8 @@ int stack_create(const tgx_stack_desc* desc, const tgx_layer_desc* layers, int d
   while ((1 << sm->page_shift) < page) sm->page_shift++;
   // what the shared sampler / token rings read from the flat description
   c->d.family = d.family; c->d.hidden = d.width; c->d.layers = d.layers; c->d.vocab = d.vocab; c->d.max_ctx = d.max_ctx; c->d.max_batch = d.max_seqs;
-  c->d.compute_dtype = d.compute_dtype; c->d.tied = 1; c->d.norm_eps = d.norm_eps;
+  c->d.compute_dtype = d.compute_dtype; c->d.tied = sandwich ? 0 : 1; c->d.norm_eps = d.norm_eps;
+  sm->sandwich = sandwich;
   c->device = device_ordinal;
   c->dt = d.compute_dtype == TGX_BF16 ? tgx::DT_BF16 : (d.compute_dtype == TGX_F16 ? tgx::DT_F16 : tgx::DT_F32);
   c->esz = d.compute_dtype == TGX_F32 ? 4 : 2;
@@ -417,6 +775,7 @@ int stack_create(const tgx_stack_desc* desc, const tgx_layer_desc* layers, int d
   if ((rc = dev_alloc(c, &c->embed, (size_t)d.vocab * W * es)) || (rc = dev_alloc(c, &sm->final_norm, W))) return rc;
   sm->missing.insert("embed"); sm->missing.insert("final.norm");
   sm->L.resize((size_t)d.layers);
+  if (sandwich) return create_sandwich_layers(c, layers);
   for (int i = 0; i < d.layers; i++) {
     StackLayerW& w = sm->L[(size_t)i];
     w.d = layers[i];
@@ -455,6 +814,7 @@ int stack_upload(tgx_ctx* c, const char* name, const void* host, const int64_t* 
   const bool probe = nd < 0;      // name lookup only (include/tgx.h): every tensor this model knows is a parameter it needs
   auto done = [&](int rc) { if (!rc) sm->missing.erase(name); return rc; };
   if (src_dtype != TGX_BF16 && src_dtype != TGX_F32 && src_dtype != TGX_F16) return set_err(c, TGX_ERR_INVALID, "unknown source dtype %d", src_dtype);
+  if (sm->sandwich) return upload_sandwich(c, name, host, shape, nd, src_dtype);
   if (!strcmp(name, "embed")) { if (probe) return TGX_ERR_SHAPE; if (!is(d.vocab, W)) return bad_shape(); return done(upload_param_ext(c, c->embed, host, d.vocab * W, src_dtype)); }
   if (!strcmp(name, "final.norm")) { if (probe) return TGX_ERR_SHAPE; if (!is(W, -1)) return bad_shape(); return done(upload_f32(c, sm->final_norm, host, W, src_dtype)); }
   int li = -1;
@@ -518,10 +878,12 @@ int stack_finalize(tgx_ctx* c) {
   const size_t W = (size_t)d.width, B = (size_t)d.max_seqs, V = (size_t)d.vocab;
   int rc;
   // angles of the position vector: pos * base^(-2i / width), the factor rounded to fp32 once
-  std::vector<float> fq(W / 2 + 1);
-  for (size_t i = 0; i < fq.size(); i++) fq[i] = (float)pow(10000.0, -2.0 * (double)i / (double)W);
-  if ((rc = dev_alloc(c, &sm->freq, fq.size()))) return rc;
-  HIP_OK(c, hipMemcpy(sm->freq, fq.data(), fq.size() * 4, hipMemcpyHostToDevice));
+  if (!sm->sandwich) {
+    std::vector<float> fq(W / 2 + 1);
+    for (size_t i = 0; i < fq.size(); i++) fq[i] = (float)pow(10000.0, -2.0 * (double)i / (double)W);
+    if ((rc = dev_alloc(c, &sm->freq, fq.size()))) return rc;
+    HIP_OK(c, hipMemcpy(sm->freq, fq.data(), fq.size() * 4, hipMemcpyHostToDevice));
+  }
   // the latent pool and its page tables
   const long long budget = d.budget_tokens > 0 ? d.budget_tokens : (long long)d.max_seqs * d.max_ctx;
   sm->n_pages = (int)((budget + sm->page - 1) / sm->page);
@@ -532,8 +894,33 @@ int stack_finalize(tgx_ctx* c) {
   memset(sm->tbl_host, 0, B * (size_t)sm->tbl_stride * 4);
   sm->row_pages.assign(B, 0); sm->row_par.assign(B, 0); sm->row_dirty.assign(B, 0);
   for (int p = sm->n_pages - 1; p >= 0; p--) sm->free_pages.push_back(p);
-  const size_t nb = (size_t)d.canon_taps - 1;
+  const size_t nb = sm->sandwich ? 0 : (size_t)d.canon_taps - 1;
+  for (auto& r : sm->rot) {      // angle of (position, pair i) = position * base^(-2i / dims), evaluated in double, stored as fp32 cosine and sine
+    const size_t half = (size_t)r.dims / 2;
+    std::vector<float> cs((size_t)d.max_ctx * half * 2);
+    for (size_t i = 0; i < half; i++) {
+      const double f = pow((double)r.base, -2.0 * (double)i / (double)r.dims);
+      for (size_t p = 0; p < (size_t)d.max_ctx; p++) { cs[(p * half + i) * 2] = (float)cos((double)p * f); cs[(p * half + i) * 2 + 1] = (float)sin((double)p * f); }
+    }
+    if ((rc = dev_alloc(c, &r.cs, cs.size()))) return rc;
+    HIP_OK(c, hipMemcpy(r.cs, cs.data(), cs.size() * 4, hipMemcpyHostToDevice));
+  }
   for (auto& w : sm->L) {
+    if (sm->sandwich) {
+      if (w.d.mixer == TGX_MIXER_ATTENTION) {      // keys and values of the layer, one page table for both
+        const size_t ke = (size_t)sm->n_pages * sm->page * (size_t)w.d.kv_heads * w.d.dim * c->esz, ve = (size_t)sm->n_pages * sm->page * (size_t)w.d.kv_heads * w.d.vdim * c->esz;
+        if ((rc = dev_alloc(c, &w.pool, ke)) || (rc = dev_alloc(c, &w.poolV, ve))) return rc;
+        HIP_OK(c, hipMemset(w.pool, 0, ke));
+        HIP_OK(c, hipMemset(w.poolV, 0, ve));
+      } else {                                     // the recurrent state of every slot (a sequence's first token starts from zero whatever the slot held)
+        const size_t hs = B * (size_t)w.d.heads;
+        if ((rc = dev_alloc(c, &w.mS, hs * w.d.dim * w.d.vdim)) || (rc = dev_alloc(c, &w.mn, 2 * hs * w.d.dim)) || (rc = dev_alloc(c, &w.mm, 2 * hs))) return rc;
+        HIP_OK(c, hipMemset(w.mS, 0, hs * w.d.dim * w.d.vdim * 4));
+        HIP_OK(c, hipMemset(w.mn, 0, 2 * hs * w.d.dim * 4));
+        HIP_OK(c, hipMemset(w.mm, 0, 2 * hs * 4));
+      }
+      continue;
+    }
     const size_t pe = (size_t)sm->n_pages * sm->page * (size_t)w.d.kv_rank * c->esz;
     if ((rc = dev_alloc(c, &w.pool, pe))) return rc;
     HIP_OK(c, hipMemset(w.pool, 0, pe));
@@ -587,7 +974,10 @@ void stack_destroy(tgx_ctx* c) {
   for (auto& w : sm->L) {
     fr(w.norm1); fr(w.norm2); fr(w.canon1); fr(w.canon2); fr(w.dwa); fr(w.w_in); fr(w.w_ukT); fr(w.w_uv); fr(w.w_o); fr(w.lat_norm); fr(w.sink);
     fr(w.w_gate); fr(w.w_up); fr(w.w_down); fr(w.w_router); fr(w.b_router); fr(w.pool); fr(w.poolT); fr(w.conv_state);
+    fr(w.b_in); fr(w.poolV); fr(w.vmix); fr(w.head_w); fr(w.mS); fr(w.mn); fr(w.mm); fr(w.act); fr(w.ws_gate); fr(w.ws_up); fr(w.ws_down);
   }
+  for (auto& r : sm->rot) fr(r.cs);
+  fr(sm->head); fr(sm->norm_g); fr(sm->a2); fr(sm->ytmp); fr(sm->ysh); fr(sm->sgw); fr(sm->vfirst); fr(sm->hs);
   fr(sm->final_norm); fr(sm->freq); fr(sm->tbl_dev); fr(sm->meta_dev); fr(sm->x); fr(sm->xs); fr(sm->a); fr(sm->proj); fr(sm->ql); fr(sm->lat); fr(sm->o); fr(sm->selw);
   fr(sm->yh); fr(sm->yd); fr(sm->xn); fr(sm->lg); fr(sm->part); fr(sm->zr); fr(sm->sel); fr(sm->moe_off); fr(sm->perm); fr(sm->ptok); fr(sm->tile_e); fr(sm->tile_m0); fr(sm->n_tiles);
   if (sm->tbl_host) (void)hipHostFree(sm->tbl_host);
@@ -746,7 +1136,8 @@ int stack_read_latent(tgx_ctx* c, int row, int layer, float* out) {
   if (row < 0 || row >= sm->d.max_seqs || layer < 0 || layer >= sm->d.layers || !out) return set_err(c, TGX_ERR_INVALID, "read_kv: row / layer out of range");
   HIP_OK(c, hipStreamSynchronize(c->stream));
   const StackLayerW& w = sm->L[(size_t)layer];
-  const size_t R = (size_t)w.d.kv_rank;
+  if (sm->sandwich && w.d.mixer != TGX_MIXER_ATTENTION) return set_err(c, TGX_ERR_UNSUPPORTED, "read_kv: layer %d caches no rows (its state is recurrent)", layer);
+  const size_t R = sm->sandwich ? (size_t)w.d.kv_heads * w.d.dim : (size_t)w.d.kv_rank;      // an attention layer's cached keys, all key heads of a token in a row
   std::vector<unsigned char> buf(R * c->esz);
   for (int64_t t = 0; t < c->row_past[(size_t)row]; t++) {
     const size_t page = (size_t)sm->tbl_host[(size_t)row * sm->tbl_stride + (size_t)(t >> sm->page_shift)];
@@ -762,9 +1153,17 @@ int64_t stack_bytes_per_token(const tgx_ctx* c, int64_t T) {
   const StackModel* sm = c->stack;
   const int64_t W = sm->d.width, es = (int64_t)c->esz;
   int64_t b = (int64_t)sm->d.vocab * W * es;
+  if (sm->sandwich) b *= 2;      // embedding row aside, the head is a matrix of its own
   for (const auto& w : sm->L) {
     const tgx_layer_desc& l = w.d;
     const int64_t H = l.heads, qd = H * l.dim, R = l.kv_rank, vd = H * l.vdim;
+    if (sm->sandwich) {
+      if (l.mixer == TGX_MIXER_ATTENTION) b += ((qd + (int64_t)l.kv_heads * (l.dim + l.vdim) + vd) * W + W * vd) * es + T * l.kv_heads * (l.dim + l.vdim) * es;
+      else b += ((2 * qd + 2 * vd + 2 * H) * W + W * vd) * es + 2 * H * (int64_t)l.dim * l.vdim * 4;      // the state is read and written
+      if (l.mlp == TGX_MLP_DENSE) b += 2 * (int64_t)l.ff * W * es;
+      if (l.mlp == TGX_MLP_MOE) b += (int64_t)(l.experts + l.identity + 1) * W * 4 + (int64_t)std::min(l.top, l.experts) * 3 * l.ff * W * es + (int64_t)3 * l.shared_ff * W * es;
+      continue;
+    }
     b += ((qd + R + vd) * W + qd * R + vd * R + W * vd) * es + T * R * es;
     if (l.mlp == TGX_MLP_MOE) b += (int64_t)l.experts * W * 4 + (int64_t)l.top * 3 * l.ff * W * es;
   }

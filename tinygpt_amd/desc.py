@@ -269,15 +269,22 @@ def known_desc(key: str, compute_dtype: str | None = None, max_batch: int = 1) -
 
 # ---- layered models (include/tgx.h tgx_stack_desc / tgx_layer_desc) -------------------------------------------------------------
 FAMILY_ZAKUSUN = 6
-MIXER_BY_NAME = {"latent_attention": 1}
-MLP_BY_NAME = {None: 0, "moe": 1}
+FAMILY_MODEPEL = 7
+STACK_FAMILY = {"zakusun": FAMILY_ZAKUSUN, "modepel": FAMILY_MODEPEL}
+MIXER_BY_NAME = {"latent_attention": 1, "attention": 2, "mlstm": 3}
+MLP_BY_NAME = {None: 0, "moe": 1, "dense": 2}
+# which mixers a design is made of (config.json "architecture" -> layer "type")
+MIXERS_OF = {"zakusun": ("latent_attention",), "modepel": ("attention", "mlstm")}
 
 
 class CLayerDesc(ctypes.Structure):
     """ctypes image of ``struct tgx_layer_desc``."""
     _fields_ = [("mixer", ctypes.c_int32), ("heads", ctypes.c_int32), ("dim", ctypes.c_int32), ("vdim", ctypes.c_int32),
                 ("kv_rank", ctypes.c_int32), ("scale", ctypes.c_float), ("mlp", ctypes.c_int32), ("experts", ctypes.c_int32),
-                ("top", ctypes.c_int32), ("ff", ctypes.c_int32), ("limit", ctypes.c_float)]
+                ("top", ctypes.c_int32), ("ff", ctypes.c_int32), ("limit", ctypes.c_float),
+                ("kv_heads", ctypes.c_int32), ("rot_dims", ctypes.c_int32), ("rot_base", ctypes.c_float), ("v_mix", ctypes.c_int32),
+                ("gate_cap", ctypes.c_float), ("identity", ctypes.c_int32), ("groups", ctypes.c_int32), ("groups_keep", ctypes.c_int32),
+                ("router_scale", ctypes.c_float), ("shared_ff", ctypes.c_int32)]
 
 
 class CStackDesc(ctypes.Structure):
@@ -301,15 +308,30 @@ class LayerDesc:
     top: int = 0
     ff: int = 0
     limit: float = 0.0
+    # grouped-query attention (mixer "attention")
+    kv_heads: int = 0
+    rot_dims: int = 0
+    rot_base: float = 10000.0
+    v_mix: bool = False
+    # matrix memory (mixer "mlstm")
+    gate_cap: float = 0.0
+    # grouped-choice experts (Modepel's "moe"): router outputs beyond `experts` hand the input through
+    identity: int = 0
+    groups: int = 1
+    groups_keep: int = 1
+    router_scale: float = 1.0
+    shared_ff: int = 0
 
     def to_c(self) -> CLayerDesc:
         return CLayerDesc(MIXER_BY_NAME[self.mixer], self.heads, self.dim, self.vdim, self.kv_rank, self.scale,
-                          MLP_BY_NAME[self.mlp], self.experts, self.top, self.ff, self.limit)
+                          MLP_BY_NAME[self.mlp], self.experts, self.top, self.ff, self.limit,
+                          self.kv_heads, self.rot_dims, self.rot_base, int(self.v_mix), self.gate_cap, self.identity, self.groups,
+                          self.groups_keep, self.router_scale, self.shared_ff)
 
 
 @dataclass
 class StackDesc:
-    """A model described layer by layer (Zakusun): the Python mirror of tgx_stack_desc + its tgx_layer_desc array."""
+    """A model described layer by layer (Zakusun, Modepel): the Python mirror of tgx_stack_desc + its tgx_layer_desc array."""
     family: str = "zakusun"
     width: int = 0
     vocab: int = 0
@@ -334,7 +356,7 @@ class StackDesc:
 
     def to_c(self):
         arr = (CLayerDesc * len(self.layers))(*[l.to_c() for l in self.layers])
-        sd = CStackDesc(FAMILY_ZAKUSUN, self.width, len(self.layers), self.vocab, DTYPE_BY_NAME[self.compute_dtype], self.max_seqs,
+        sd = CStackDesc(STACK_FAMILY[self.family], self.width, len(self.layers), self.vocab, DTYPE_BY_NAME[self.compute_dtype], self.max_seqs,
                         self.max_ctx, self.budget_tokens, self.page_tokens, self.norm_groups, self.norm_eps, self.canon_taps,
                         self.logit_scale)
         return sd, arr
@@ -343,6 +365,8 @@ class StackDesc:
         """checkpoint name -> shape, in file order"""
         W, out = self.width, {}
         out["embed"] = (self.vocab, W)
+        if self.family == "modepel":
+            return self._modepel_shapes(out)
         for i, l in enumerate(self.layers):
             p = f"l{i}."
             out[p + "norm1"] = (W,)
@@ -363,10 +387,75 @@ class StackDesc:
         return out
 
 
+    def _modepel_shapes(self, out):
+        W = self.width
+        for i, l in enumerate(self.layers):
+            p = f"l{i}."
+            for n in ("norm1", "norm2", "norm1b", "norm2b") if l.mlp else ("norm1", "norm1b"):
+                out[p + n] = ()
+            qd, vd = l.heads * l.dim, l.heads * l.vdim
+            if l.mixer == "attention":
+                kd, kv = l.kv_heads * l.dim, l.kv_heads * l.vdim
+                out[p + "mix.q"] = (qd, W); out[p + "mix.q.b"] = (qd,); out[p + "mix.k"] = (kd, W); out[p + "mix.k.b"] = (kd,)
+                out[p + "mix.v"] = (kv, W); out[p + "mix.v.b"] = (kv,)
+                if l.v_mix:
+                    out[p + "mix.vmix"] = ()
+                out[p + "mix.g"] = (vd, W); out[p + "mix.o"] = (W, vd)
+            else:
+                out[p + "mix.q"] = (qd, W); out[p + "mix.k"] = (qd, W); out[p + "mix.v"] = (vd, W); out[p + "mix.g"] = (vd, W); out[p + "mix.o"] = (W, vd)
+                out[p + "mix.norm"] = (vd,); out[p + "mix.i"] = (l.heads, W); out[p + "mix.i.b"] = (l.heads,)
+                out[p + "mix.f"] = (l.heads, W); out[p + "mix.f.b"] = (l.heads,)
+            if l.mlp == "dense":
+                out[p + "mlp.up"] = (l.ff, W); out[p + "mlp.down"] = (W, l.ff); out[p + "mlp.act"] = (4,)
+            elif l.mlp == "moe":
+                for e in range(l.experts):
+                    out[p + f"mlp.e{e}.gate"] = (l.ff, W); out[p + f"mlp.e{e}.up"] = (l.ff, W); out[p + f"mlp.e{e}.down"] = (W, l.ff)
+                out[p + "mlp.router"] = (l.experts + l.identity, W); out[p + "mlp.correction"] = (l.experts + l.identity,)
+                if l.shared_ff:
+                    out[p + "mlp.shared.gate"] = (l.shared_ff, W); out[p + "mlp.shared.up"] = (l.shared_ff, W)
+                    out[p + "mlp.shared.down"] = (W, l.shared_ff); out[p + "mlp.shared.sg"] = (1, W)
+        out["final.norm"] = ()
+        out["head"] = (self.vocab, W)
+        return out
+
+
+def _modepel_layer(i: int, l: dict) -> LayerDesc:
+    """one entry of a Modepel config's "layers": {"type": "attention" | "mlstm", "mixer": {...}, "mlp": null | {"kind": "dense" | "moe", ...}}"""
+    m, f = l["mixer"], l.get("mlp")
+    ld = LayerDesc(mixer=l["type"], heads=int(m["heads"]), dim=int(m["dim"]), vdim=int(m["vdim"]))
+    if l["type"] == "attention":
+        rot = m.get("rot") or {}
+        ld.kv_heads = int(m["kv_heads"]); ld.scale = float(m["scale"]); ld.v_mix = bool(m.get("v_mix", False))
+        ld.rot_dims = int(rot.get("dims", 0)); ld.rot_base = float(rot.get("base", 10000.0))
+    else:
+        ld.gate_cap = float(m["gate_cap"])
+    if f is None:
+        return ld
+    if f.get("kind") == "dense":
+        ld.mlp = "dense"; ld.ff = int(f["ff"])
+    elif f.get("kind") == "moe":
+        r, g = f["router"], f["router"].get("groups") or {}
+        ld.mlp = "moe"; ld.experts = int(r["experts"]); ld.identity = int(r.get("identity", 0)); ld.top = int(r["top"])
+        ld.router_scale = float(r.get("scale", 1.0)); ld.groups = int(g.get("count", 1)); ld.groups_keep = int(g.get("keep", ld.groups))
+        ld.ff = int(f["expert"]["ff"]) if ld.experts else 0
+        ld.shared_ff = int(f["shared"]["ff"]) if f.get("shared") else 0
+    else:
+        raise ValueError(f"layer {i}: feed-forward kind {f.get('kind')!r} is not implemented")
+    return ld
+
+
 def stack_desc_from_config(cfg: dict, compute_dtype: str = "bf16", max_seqs: int = 4, max_ctx: int = 4096, budget_tokens: int = 0) -> StackDesc:
-    """config.json of a layered model ("architecture": "Zakusun") -> StackDesc.  Every size and constant comes from the file."""
-    if cfg.get("architecture") != "Zakusun":
+    """config.json of a layered model ("architecture": "Zakusun" | "Modepel") -> StackDesc.  Every size and constant comes from the file."""
+    arch = str(cfg.get("architecture")).lower()
+    if arch not in MIXERS_OF:
         raise ValueError(f"Unsupported architecture: {cfg.get('architecture')!r}")
+    for i, l in enumerate(cfg["layers"]):
+        if l["type"] not in MIXERS_OF[arch]:
+            raise ValueError(f"layer {i}: mixer {l['type']!r} is not implemented")
+    if arch == "modepel":
+        return StackDesc(family="modepel", width=int(cfg["width"]), vocab=int(cfg["vocab"]), layers=[_modepel_layer(i, l) for i, l in enumerate(cfg["layers"])],
+                         compute_dtype=compute_dtype, max_seqs=max_seqs, max_ctx=max_ctx, budget_tokens=budget_tokens, norm_groups=1,
+                         norm_eps=float(cfg["norm"]["eps"]), canon_taps=1, logit_scale=1.0, name="modepel")
     layers = []
     for i, l in enumerate(cfg["layers"]):
         if l["type"] not in MIXER_BY_NAME:
