@@ -83,6 +83,7 @@ def parse():
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--layered", default=None, metavar="SIZE[,SIZE]", help="instead of the headline: prefill and decode throughput of the layered (Zakusun) design at "
                     "layer sizes of real models (1b, 0.5b; random weights), beside a Llama-family model of the same width, depth and active parameters")
+    ap.add_argument("--design", default="zakusun", choices=["zakusun", "modepel"], help="with --layered: which layered design is measured beside the Llama-family model")
     ap.add_argument("--cpu-seconds", type=float, default=15.0, help="target CPU time of the cpu_baseline sample")
     return ap.parse_args()
 
@@ -312,6 +313,25 @@ LAYERED_SIZES = {
 }
 
 
+def modepel_desc(key, z, L, V, dtype, B, ctx):
+    """Modepel at the size of `z`: mLSTM layers (value heads twice as wide as key heads) at every third place, grouped-query attention with rotary positions,
+    value mixing and a sink elsewhere; a dense PolyNorm feed-forward in the first layer, grouped-choice experts (identity outputs, a shared expert) in the others"""
+    from tinygpt_amd.desc import LayerDesc, StackDesc
+    W = z["width"]
+    layers = []
+    for i in range(L):
+        if i % 3 == 0:
+            l = LayerDesc(mixer="mlstm", heads=W // 256, dim=128, vdim=256, gate_cap=15.0)
+        else:
+            l = LayerDesc(mixer="attention", heads=W // 128, kv_heads=max(1, W // 512), dim=128, vdim=128, rot_dims=64, rot_base=500000.0, scale=128 ** -0.5, v_mix=True)
+        if i == 0:
+            l.mlp, l.ff = "dense", z["top"] * z["ff"]
+        else:
+            l.mlp, l.experts, l.identity, l.top, l.ff, l.groups, l.groups_keep, l.router_scale, l.shared_ff = "moe", z["experts"], z["experts"] // 4, z["top"], z["ff"], 4, 2, 1.5, z["ff"]
+        layers.append(l)
+    return StackDesc(family="modepel", width=W, vocab=V, compute_dtype=dtype, max_seqs=B, max_ctx=ctx, budget_tokens=B * (ctx + 64), norm_eps=1e-5, name=f"modepel-{key}", layers=layers)
+
+
 def layered_compare(args):
     from tinygpt_amd.desc import LayerDesc, ModelDesc, StackDesc
     from tinygpt_amd.ffi import GREEDY, Model
@@ -357,14 +377,14 @@ def layered_compare(args):
                                          top=z["top"], ff=z["ff"], limit=7.0) for _ in range(L)])
         ld = ModelDesc(family="llama", hidden=z["width"], layers=L, heads=z["llama"]["heads"], kv_heads=z["llama"]["kv_heads"], head_dim=z["width"] // z["llama"]["heads"],
                        inter=z["llama"]["inter"], vocab=V, max_ctx=ctx, tied=True, compute_dtype=args.dtype, norm_eps=1e-5, rope_theta=500000.0, max_batch=B, name=f"llama-{key}")
-        for desc, layered in ((sd, True), (ld, False)):
+        for desc, layered in ([(modepel_desc(key, z, L, V, args.dtype, B, ctx), True)] if args.design == "modepel" else []) + [(sd, True), (ld, False)]:
             m = Model(desc).load_synthetic(1234, 0.02).finalize()
             r = measure(m, layered)
             m.close()
             r["model"] = desc.name
             rows.append(r)
             print(json.dumps(r), file=sys.stderr, flush=True)
-    print(json.dumps({"metric": "layered_vs_flat_throughput", "unit": "tokens/s", "dtype": args.dtype, "data": "synthetic", "prompt": S, "layers": L, "vocab": V,
+    print(json.dumps({"metric": "layered_vs_flat_throughput", "design": args.design, "unit": "tokens/s", "dtype": args.dtype, "data": "synthetic", "prompt": S, "layers": L, "vocab": V,
                       "decode_steps": ND, "rows": rows}))
 
 

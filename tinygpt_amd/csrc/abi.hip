@@ -511,7 +511,7 @@ int tgx_create_stack(const tgx_stack_desc* desc, const tgx_layer_desc* layers, i
 }
 
 int tgx_upload(tgx_ctx* c, const char* name, const void* host, const int64_t* shape, int nd, int src_dtype) {
-  if (!c || !name || !host || !shape) return c ? set_err(c, TGX_ERR_INVALID, "null argument") : TGX_ERR_INVALID;
+  if (!c || !name || !host || (!shape && nd != 0)) return c ? set_err(c, TGX_ERR_INVALID, "null argument") : TGX_ERR_INVALID;      // (a tensor of one number has no shape entries)
   HIP_OK(c, hipSetDevice(c->device));
   if (c->stack) return stack_upload(c, name, host, shape, nd, src_dtype);
   const tgx_model_desc& d = c->d;

@@ -52,34 +52,78 @@ static bool check_dims(const tgx_model_desc& d, const std::string& path, std::st
   return true;
 }
 
+// one entry of a Modepel config's "layers": {"type": "attention" | "mlstm", "mixer": {...}, "mlp": null | {"kind": "dense" | "moe", ...}}
+static bool load_modepel_layer(const Json& L, size_t i, tgx_layer_desc& l, std::string& err) {
+  auto dim = [](const Json& j, const char* key) -> int32_t { const int64_t v = j.get_int(key, -1); return (v < 0 || v > ((int64_t)1 << 30)) ? -1 : (int32_t)v; };
+  const Json* mx = L.get("mixer");
+  const Json* ff = L.get("mlp");
+  const std::string type = L.get_str("type", "");
+  if ((type != "attention" && type != "mlstm") || !mx || mx->kind != Json::Obj) { err = "config.json: layer " + std::to_string(i) + ": mixer '" + type + "' is not implemented"; return false; }
+  l.heads = dim(*mx, "heads"); l.dim = dim(*mx, "dim"); l.vdim = dim(*mx, "vdim");
+  if (type == "attention") {
+    l.mixer = TGX_MIXER_ATTENTION;
+    l.kv_heads = dim(*mx, "kv_heads"); l.scale = mx->get_float("scale", 1.f);
+    const Json* vm = mx->get("v_mix");
+    l.v_mix = vm && vm->kind == Json::Bool && vm->b ? 1 : 0;
+    const Json* rot = mx->get("rot");
+    if (rot && rot->kind == Json::Obj) { l.rot_dims = dim(*rot, "dims"); l.rot_base = rot->get_float("base", 10000.f); }
+  } else {
+    l.mixer = TGX_MIXER_MLSTM;
+    l.gate_cap = mx->get_float("gate_cap", 0.f);
+  }
+  if (!ff || ff->kind != Json::Obj) return true;
+  const std::string kind = ff->get_str("kind", "");
+  if (kind == "dense") { l.mlp = TGX_MLP_DENSE; l.ff = dim(*ff, "ff"); return true; }
+  const Json* ex = ff->get("expert");
+  const Json* ro = ff->get("router");
+  if (kind != "moe" || !ro || ro->kind != Json::Obj) { err = "config.json: layer " + std::to_string(i) + ": feed-forward kind '" + kind + "' is not implemented"; return false; }
+  l.mlp = TGX_MLP_MOE;
+  l.experts = dim(*ro, "experts"); l.top = dim(*ro, "top"); l.router_scale = ro->get_float("scale", 1.f);
+  l.identity = ro->has("identity") ? dim(*ro, "identity") : 0;
+  const Json* gr = ro->get("groups");
+  l.groups = 1; l.groups_keep = 1;
+  if (gr && gr->kind == Json::Obj) { l.groups = dim(*gr, "count"); l.groups_keep = gr->has("keep") ? dim(*gr, "keep") : l.groups; }
+  l.ff = l.experts > 0 && ex && ex->kind == Json::Obj ? dim(*ex, "ff") : 0;
+  const Json* sh = ff->get("shared");
+  l.shared_ff = sh && sh->kind == Json::Obj ? dim(*sh, "ff") : 0;
+  return true;
+}
+
 // config.json of a layered model: {"architecture": "Zakusun", "width", "vocab", "logit_scale", "norm": {"eps", "groups"}, "canon": {"taps"},
 // "layers": [{"type": mixer, "mixer": {heads, dim, vdim, kv_rank, scale}, "mlp": null | {"kind": "moe", "expert": {ff, limit}, "router": {experts, top}}}]}
+// or {"architecture": "Modepel", "width", "vocab", "norm": {"eps"}, "layers": [...]} with the layer entries of load_modepel_layer
 static bool load_stack_config(const Json& doc, const std::string& path, int compute_dtype, int max_batch, int max_ctx, int budget_tokens, ModelConfig& out, std::string& err) {
   const std::string arch = doc.get_str("architecture", "");
-  if (arch != "Zakusun") { err = "Unsupported architecture: " + arch; return false; }
+  const bool modepel = arch == "Modepel";
+  if (arch != "Zakusun" && !modepel) { err = "Unsupported architecture: " + arch; return false; }
   auto dim = [](const Json& j, const char* key) -> int32_t { const int64_t v = j.get_int(key, -1); return (v < 0 || v > ((int64_t)1 << 30)) ? -1 : (int32_t)v; };
   out.layered = true;
-  out.model_type = "zakusun";
+  out.model_type = modepel ? "modepel" : "zakusun";
   tgx_stack_desc& s = out.stack;
-  s.family = TGX_FAMILY_ZAKUSUN;
+  s.family = modepel ? TGX_FAMILY_MODEPEL : TGX_FAMILY_ZAKUSUN;
   s.width = dim(doc, "width"); s.vocab = dim(doc, "vocab"); s.compute_dtype = compute_dtype;
   s.max_seqs = max_batch < 1 ? 1 : max_batch;
   s.max_ctx = max_ctx > 0 ? max_ctx : 4096;
   s.budget_tokens = budget_tokens > 0 ? budget_tokens : 0;
   s.page_tokens = 0;
-  s.logit_scale = doc.get_float("logit_scale", 1.f);
+  s.logit_scale = modepel ? 1.f : doc.get_float("logit_scale", 1.f);
   const Json* norm = doc.get("norm");
   const Json* canon = doc.get("canon");
   const Json* layers = doc.get("layers");
-  if (!norm || norm->kind != Json::Obj || !canon || canon->kind != Json::Obj || !layers || layers->kind != Json::Arr || layers->arr.empty()) {
+  if (!norm || norm->kind != Json::Obj || (!modepel && (!canon || canon->kind != Json::Obj)) || !layers || layers->kind != Json::Arr || layers->arr.empty()) {
     err = "config.json: norm / canon / layers are missing in " + path; return false;
   }
-  s.norm_groups = dim(*norm, "groups"); s.norm_eps = norm->get_float("eps", 1e-6f); s.canon_taps = dim(*canon, "taps");
+  s.norm_groups = modepel ? 1 : dim(*norm, "groups"); s.norm_eps = norm->get_float("eps", 1e-6f); s.canon_taps = modepel ? 1 : dim(*canon, "taps");
   for (size_t i = 0; i < layers->arr.size(); i++) {
     const Json& L = layers->arr[i];
+    tgx_layer_desc l{};
+    if (modepel) {
+      if (!load_modepel_layer(L, i, l, err)) return false;
+      out.layers.push_back(l);
+      continue;
+    }
     const Json* mx = L.get("mixer");
     const Json* ff = L.get("mlp");
-    tgx_layer_desc l{};
     const std::string type = L.get_str("type", "");
     if (type != "latent_attention" || !mx || mx->kind != Json::Obj) { err = "config.json: layer " + std::to_string(i) + ": mixer '" + type + "' is not implemented"; return false; }
     l.mixer = TGX_MIXER_LATENT_ATTENTION;
@@ -95,7 +139,7 @@ static bool load_stack_config(const Json& doc, const std::string& path, int comp
   }
   s.layers = (int32_t)out.layers.size();
   tgx_model_desc& d = out.desc;
-  d.family = s.family; d.hidden = s.width; d.layers = s.layers; d.vocab = s.vocab; d.max_ctx = s.max_ctx; d.max_batch = s.max_seqs; d.compute_dtype = compute_dtype; d.tied = 1;
+  d.family = s.family; d.hidden = s.width; d.layers = s.layers; d.vocab = s.vocab; d.max_ctx = s.max_ctx; d.max_batch = s.max_seqs; d.compute_dtype = compute_dtype; d.tied = modepel ? 0 : 1;
   if (s.width <= 0 || s.vocab <= 0 || s.norm_groups <= 0 || s.canon_taps <= 0) { err = "config.json: width / vocab / norm.groups / canon.taps missing or out of range in " + path; return false; }
   return true;
 }
