@@ -415,3 +415,32 @@ def test_what_the_library_refuses():
     with pytest.raises(TgxError, match="l0.mix.f.b"):
         m.finalize()
     m.close()
+
+
+# ---- attention on the matrix cores (16-bit storage; key sizes 64 / 128 / 256, value sizes in steps of 32) --------------------------------------
+@pytest.mark.parametrize("heads,kv,dim,vdim", [(4, 1, 64, 32), (8, 2, 128, 128), (6, 3, 64, 96), (2, 2, 128, 256), (16, 4, 64, 64), (3, 1, 256, 192)])
+def test_matrix_core_attention_equals_the_lane_kernel(heads, kv, dim, vdim):
+    """the same bf16 weights and cached rows through both attention kernels: portions whose 32-row tiles cut through tokens, a mixed batch, decoding,
+    contexts across page borders, and the split-keys form.  The two differ by summation order and the two-term rounding of q and p only."""
+    mixer = dict(heads=heads, kv_heads=kv, dim=dim, vdim=vdim, rot={"dims": 32, "base": 10000.0}, scale=1.2 * dim ** -0.5)
+    cfg = config([attn(**mixer), attn(moe(), **mixer)], width=64)
+    w = mo.random_tensors(cfg, heads)
+    tens = {k: np.asarray(v, np.float32) for k, v in w.items()}
+    mk = lambda: SlotEngine(desc=stack_desc_from_config(cfg, "bf16", max_seqs=4, max_ctx=1024, budget_tokens=2048), tensors=tens)
+    fast, slow = mk(), mk()
+    slow.model.set_option("attn.mfma", 0)
+    a, b, c = tokens(cfg, 200, 1), tokens(cfg, 75, 2), tokens(cfg, 9, 3)
+    want = want_of(cfg, w, a)[[0, 1, 69, 130, 131, 199]]
+    outs = []
+    for eng in (fast, slow):
+        o = [eng.step([("a", a[:70], [0, 1, 69]), ("b", b[:3], [2])])]
+        o.append(eng.step([("a", a[70:131], [60]), ("c", c, [8]), ("b", b[3:4], [0])]))
+        o.append(eng.step([("b", b[4:], [70]), ("a", a[131:132], [0])]))
+        o.append(eng.step([("a", a[132:199], [])]))
+        eng.model.set_option("attn.split_min", 64)
+        o.append(eng.step([("a", a[199:], [0]), ("b", [5], [0])]))
+        outs.append(np.concatenate(o))
+    assert np.abs(outs[0] - outs[1]).max() / np.abs(outs[1]).max() < 3e-4
+    check(outs[0][[0, 1, 2, 4, 8, 9]], want, "bf16")               # a's positions 0, 1, 69, 130, 131, 199 in the order the steps returned them
+    check(outs[0][[6, 7]], want_of(cfg, w, b)[[3, 74]], "bf16")
+    fast.close(); slow.close()

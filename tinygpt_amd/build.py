@@ -24,7 +24,7 @@ FLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-shared", "-fvi
          ] + (["-mllvm", "-amdgpu-mfma-vgpr-form"] if os.environ.get("TGX_VGPR_FORM", "1") == "1" else [])
 
 
-TUS = ["abi", "decode", "attn", "sampler", "prefill", "prefill_f32", "skinny", "stack"]     # csrc/<name>.hip, compiled in parallel (csrc/ctx.h lists what each holds)
+TUS = ["abi", "decode", "attn", "sampler", "prefill", "prefill_f32", "skinny", "stack", "stack_gqa"]     # csrc/<name>.hip, compiled in parallel (csrc/ctx.h lists what each holds)
 OBJDIR = os.path.join(LIBDIR, "obj")
 
 

@@ -6,7 +6,8 @@
 //   prefill.hip      batched MFMA prefill, 16-bit storage (kernels/prefill.h, gemm_dma.h)
 //   prefill_f32.hip  batched prefill, fp32 storage (kernels/gemm_f32.h)
 //   skinny.hip       batched decode step / short prompts on the skinny MFMA GEMMs (kernels/skinny*.h)
-//   stack.hip        layered models (tgx_create_stack): ragged engine step, paged latent cache, slot state (kernels/stack*.h)
+//   stack.hip        layered models (tgx_create_stack): ragged engine step, paged latent / key-value cache, slot state (kernels/stack*.h)
+//   stack_gqa.hip    their grouped-query attention on the matrix cores (kernels/stack_gqa_mfma.h)
 // One context = one GPU = one HIP stream; every call comes from one host thread.  There is NO CPU path in this library.
 #pragma once
 #include <hip/hip_runtime.h>

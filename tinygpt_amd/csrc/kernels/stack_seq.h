@@ -108,6 +108,7 @@ struct GqaAppendArgs {
   const float* cs;           // [positions][rot_dims / 2][2]
   void* poolK;               // [pages][page_tokens][kv_heads * dim]
   void* poolV;               // [pages][page_tokens][kv_heads * vdim]
+  void* poolVT;              // [pages][kv_heads * vdim][page_tokens]: the same values, token-contiguous per channel (nullptr: not kept)
   float* vfirst;             // [T][kv_heads * vdim] values of the first mixing layer for the step's tokens
   int vmode;                 // 0: no mixing; 1: this layer's values become vfirst; 2: v <- (1 - lam) v + lam vfirst
   const float* lam;
@@ -139,7 +140,9 @@ __global__ __launch_bounds__(256) void gqa_append_kernel(StepMeta m, GqaAppendAr
     float v = vsrc[c];
     if (a.vmode == 1) a.vfirst[(size_t)t * vd + c] = v;
     if (a.vmode == 2) v = fmaf(lam, a.vfirst[(size_t)t * vd + c], __fmul_rn(1.0f - lam, v));
-    vdst[c] = f32_to_elem<DT>(v);
+    const elem_t<DT> sv = f32_to_elem<DT>(v);
+    vdst[c] = sv;
+    if (a.poolVT) reinterpret_cast<elem_t<DT>*>(a.poolVT)[((((size_t)page * vd) + c) << m.page_shift) + (size_t)(pos & ((1 << m.page_shift) - 1))] = sv;
   }
 }
 

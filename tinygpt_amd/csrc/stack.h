@@ -27,6 +27,7 @@ struct StackLayerW {
   // grouped-query attention: w_in = [q | k | v | gate] rows, bias b_in over the same rows; mLSTM: w_in = [q | k | v | gate | zi | zf]
   float* b_in = nullptr;        // fp32 [rows of w_in]
   ebyte* poolV = nullptr;       // attention: values [pages][page_tokens][kv_heads * vdim] (`pool` holds the keys [..][kv_heads * dim])
+  ebyte* poolVT = nullptr;      // ... and their transposed copy [pages][kv_heads * vdim][page_tokens] for the matrix-core attention (layers that take it)
   float* vmix = nullptr;        // attention: the value-mixing number
   int vmode = 0;                // 0: no value mixing, 1: the first mixing layer (its values are handed on), 2: mixes
   int rot = -1;                 // index of the layer's rotation table (StackModel::rot)
@@ -73,6 +74,11 @@ struct StackModel {
   int gemv = 1;                        // option stack.gemv: 0 sends products of few rows through the matrix-core tiles as well
   int gemm_wt = 0;                     // option stack.gemm_wt: force the product's tile (1: 64 x 64, 2: 128 x 128); 0 = by the number of tiles
 };
+
+// stack_gqa.hip
+namespace tgx { struct StepMeta; struct GqaMfmaArgs; }
+bool gqa_mfma_shapes_ok(int dt, int dim, int vdim, int page_shift, long long ldq);
+void launch_gqa_mfma(tgx_ctx* c, const tgx::StepMeta& m, const tgx::GqaMfmaArgs& a, dim3 grid, bool split);
 
 int stack_create(const tgx_stack_desc* desc, const tgx_layer_desc* layers, int device_ordinal, tgx_ctx** out_ctx);
 int stack_upload(tgx_ctx* c, const char* name, const void* host, const int64_t* shape, int nd, int src_dtype);

@@ -14,6 +14,7 @@
 #include "kernels/stack_gemm.h"
 #include "kernels/stack_attn_mfma.h"
 #include "kernels/stack_seq.h"
+#include "kernels/stack_gqa_mfma.h"
 
 int upload_param_ext(tgx_ctx* c, ebyte* dst, const void* host, int64_t n, int src_dtype);      // abi.hip
 
@@ -332,7 +333,7 @@ void launch_gqa_t(tgx_ctx* c, const tgx::StepMeta& m, const tgx::GqaAttnArgs& a,
   else hipLaunchKernelGGL((tgx::gqa_attn_kernel<DT, 4, SPLIT>), grid, dim3(256), lds, c->stream, m, a);
 }
 
-int run_attention(tgx_ctx* c, const tgx::StepMeta& m, StackLayerW& w, const float* hin, int T, int max_keys) {
+int run_attention(tgx_ctx* c, const tgx::StepMeta& m, StackLayerW& w, const float* hin, int T, int S, int max_keys, int max_count) {
   StackModel* sm = c->stack;
   const tgx_layer_desc& ld = w.d;
   const int W = sm->d.width, H = ld.heads, G = ld.kv_heads, qd = H * ld.dim, kd = G * ld.dim, kvv = G * ld.vdim, vd = H * ld.vdim, nin = qd + kd + kvv + vd;
@@ -342,8 +343,34 @@ int run_attention(tgx_ctx* c, const tgx::StepMeta& m, StackLayerW& w, const floa
   launch_gemm(c, g, tgx::SG_STORE, 1);
   tgx::GqaAppendArgs ap{};
   ap.proj = sm->proj; ap.ldp = nin; ap.heads = H; ap.kv_heads = G; ap.dim = ld.dim; ap.vdim = ld.vdim; ap.rot_dims = ld.rot_dims;
-  ap.cs = w.rot >= 0 ? sm->rot[(size_t)w.rot].cs : nullptr; ap.poolK = w.pool; ap.poolV = w.poolV; ap.vfirst = sm->vfirst; ap.vmode = w.vmode; ap.lam = w.vmix;
+  ap.cs = w.rot >= 0 ? sm->rot[(size_t)w.rot].cs : nullptr; ap.poolK = w.pool; ap.poolV = w.poolV; ap.poolVT = w.poolVT; ap.vfirst = sm->vfirst; ap.vmode = w.vmode; ap.lam = w.vmix;
   TGX_DT_SWITCH(c->dt, hipLaunchKernelGGL(tgx::gqa_append_kernel<DT>, dim3(T), dim3(256), 0, c->stream, m, ap))
+  if (w.poolVT && sm->attn_mfma) {
+    // rows = (token, query head of the group) pairs of an entry and a key / value head in tiles of 32; few tiles and a long context: the keys are divided
+    tgx::GqaMfmaArgs ma{};
+    ma.q = sm->proj; ma.ldq = nin; ma.poolK = w.pool; ma.poolVT = w.poolVT; ma.gate = sm->proj + qd + kd + kvv; ma.ldg = nin; ma.out = sm->o; ma.ldo = vd;
+    ma.heads = H; ma.kv_heads = G; ma.dim = ld.dim; ma.vdim = ld.vdim; ma.terms = c->act16 ? 1 : 2; ma.scale = ld.scale; ma.sink = 0.f; ma.has_sink = 1;
+    const int tiles = (max_count * (H / G) + 31) / 32;
+    const long long wgs = (long long)tiles * S * G;
+    int nsplit = 1;
+    if (max_keys >= sm->attn_split_min_keys && wgs < c->num_cus) {
+      nsplit = (int)std::min<long long>(64, (2LL * c->num_cus) / wgs);
+      const int per = std::max(64, ((max_keys + nsplit - 1) / nsplit + 31) / 32 * 32);      // two key tiles per workgroup at least
+      nsplit = (max_keys + per - 1) / per;
+      ma.keys_per = per;
+    }
+    if (nsplit > 1) {
+      int rc = ensure_part(c, (size_t)T * H * nsplit * (size_t)(ld.vdim + 2));
+      if (rc) return rc;
+      ma.part = sm->part; ma.nsplit = nsplit;
+      launch_gqa_mfma(c, m, ma, dim3(tiles, S * G, nsplit), true);
+      tgx::GqaAttnArgs mg{};
+      mg.part = sm->part; mg.nsplit = nsplit; mg.heads = H; mg.vdim = ld.vdim; mg.gate = ma.gate; mg.ldg = nin; mg.out = sm->o; mg.ldo = vd;
+      hipLaunchKernelGGL(tgx::gqa_attn_merge_kernel, dim3(T, H), dim3(256), 0, c->stream, mg);
+    } else {
+      launch_gqa_mfma(c, m, ma, dim3(tiles, S * G), false);
+    }
+  } else {
   tgx::GqaAttnArgs aa{};
   aa.q = sm->proj; aa.ldq = nin; aa.poolK = w.pool; aa.poolV = w.poolV; aa.gate = sm->proj + qd + kd + kvv; aa.ldg = nin; aa.out = sm->o; aa.ldo = vd;
   aa.heads = H; aa.kv_heads = G; aa.dim = ld.dim; aa.vdim = ld.vdim; aa.scale = ld.scale; aa.sink = 0.f; aa.has_sink = 1;
@@ -362,6 +389,7 @@ int run_attention(tgx_ctx* c, const tgx::StepMeta& m, StackLayerW& w, const floa
     hipLaunchKernelGGL(tgx::gqa_attn_merge_kernel, dim3(T, H), dim3(256), 0, c->stream, aa);
   } else {
     TGX_DT_SWITCH(c->dt, (launch_gqa_t<DT, false>(c, m, aa, dim3(T, H))))
+  }
   }
   // y = o . w_o^T
   g = tgx::StackGemmArgs{};
@@ -447,7 +475,7 @@ void run_choice_experts(tgx_ctx* c, StackLayerW& w, const float* hin, int T) {
   }
 }
 
-int run_layers_sandwich(tgx_ctx* c, const MetaPtrs& mp, int T, int S, int max_keys) {
+int run_layers_sandwich(tgx_ctx* c, const MetaPtrs& mp, int T, int S, int max_keys, int max_count) {
   StackModel* sm = c->stack;
   const tgx::StepMeta m = step_meta(sm, mp, T, S);
   const int W = sm->d.width, L = sm->d.layers;
@@ -460,7 +488,7 @@ int run_layers_sandwich(tgx_ctx* c, const MetaPtrs& mp, int T, int S, int max_ke
     const tgx_layer_desc& ld = w.d;
     const float* ng = sm->norm_g + 4 * (size_t)li;
     const float* next_layer = li + 1 < L ? ng + 4 : nullptr;
-    int rc = ld.mixer == TGX_MIXER_ATTENTION ? run_attention(c, m, w, hin, T, max_keys) : run_mlstm(c, m, w, hin, T, S);
+    int rc = ld.mixer == TGX_MIXER_ATTENTION ? run_attention(c, m, w, hin, T, S, max_keys, max_count) : run_mlstm(c, m, w, hin, T, S);
     if (rc) return rc;
     tgx::SandwichArgs sa{};
     sa.x = sm->x; sa.y = sm->yd; sa.top = 1; sa.ytmp = sm->ytmp; sa.g_post = ng + 1; sa.g_next = ld.mlp != TGX_MLP_NONE ? ng + 2 : next_layer; sa.out = hout; sa.W = W; sa.eps = eps;
@@ -481,7 +509,7 @@ int run_layers_sandwich(tgx_ctx* c, const MetaPtrs& mp, int T, int S, int max_ke
 }
 
 int run_layers(tgx_ctx* c, const MetaPtrs& mp, int T, int S, int max_keys, int max_count) {
-  return c->stack->sandwich ? run_layers_sandwich(c, mp, T, S, max_keys) : run_layers_latent(c, mp, T, S, max_keys, max_count);
+  return c->stack->sandwich ? run_layers_sandwich(c, mp, T, S, max_keys, max_count) : run_layers_latent(c, mp, T, S, max_keys, max_count);
 }
 
 // logits of the rows listed in want_dev (indices into the step's tokens): C[crow(i)] = embed . norm(x[want[i]]) * logit_scale
@@ -912,6 +940,11 @@ int stack_finalize(tgx_ctx* c) {
         if ((rc = dev_alloc(c, &w.pool, ke)) || (rc = dev_alloc(c, &w.poolV, ve))) return rc;
         HIP_OK(c, hipMemset(w.pool, 0, ke));
         HIP_OK(c, hipMemset(w.poolV, 0, ve));
+        const long long nin = (long long)w.d.heads * (w.d.dim + w.d.vdim) + (long long)w.d.kv_heads * (w.d.dim + w.d.vdim);
+        if (gqa_mfma_shapes_ok(c->dt, w.d.dim, w.d.vdim, sm->page_shift, nin)) {
+          if ((rc = dev_alloc(c, &w.poolVT, ve))) return rc;
+          HIP_OK(c, hipMemset(w.poolVT, 0, ve));
+        }
       } else {                                     // the recurrent state of every slot (a sequence's first token starts from zero whatever the slot held)
         const size_t hs = B * (size_t)w.d.heads;
         if ((rc = dev_alloc(c, &w.mS, hs * w.d.dim * w.d.vdim)) || (rc = dev_alloc(c, &w.mn, 2 * hs * w.d.dim)) || (rc = dev_alloc(c, &w.mm, 2 * hs))) return rc;
@@ -974,7 +1007,7 @@ void stack_destroy(tgx_ctx* c) {
   for (auto& w : sm->L) {
     fr(w.norm1); fr(w.norm2); fr(w.canon1); fr(w.canon2); fr(w.dwa); fr(w.w_in); fr(w.w_ukT); fr(w.w_uv); fr(w.w_o); fr(w.lat_norm); fr(w.sink);
     fr(w.w_gate); fr(w.w_up); fr(w.w_down); fr(w.w_router); fr(w.b_router); fr(w.pool); fr(w.poolT); fr(w.conv_state);
-    fr(w.b_in); fr(w.poolV); fr(w.vmix); fr(w.head_w); fr(w.mS); fr(w.mn); fr(w.mm); fr(w.act); fr(w.ws_gate); fr(w.ws_up); fr(w.ws_down);
+    fr(w.b_in); fr(w.poolV); fr(w.poolVT); fr(w.vmix); fr(w.head_w); fr(w.mS); fr(w.mn); fr(w.mm); fr(w.act); fr(w.ws_gate); fr(w.ws_up); fr(w.ws_down);
   }
   for (auto& r : sm->rot) fr(r.cs);
   fr(sm->head); fr(sm->norm_g); fr(sm->a2); fr(sm->ytmp); fr(sm->ysh); fr(sm->sgw); fr(sm->vfirst); fr(sm->hs);
