@@ -87,6 +87,7 @@ MECH = {
     "mlstm_alone": [rec()],
     "mlstm_one_head_wide": [rec(heads=1, dim=40, vdim=70)],                  # two column chunks, rows spread over the waves
     "mlstm_large_keys": [rec(heads=2, dim=130, vdim=9)],
+    "mlstm_very_large_keys": [rec(heads=1, dim=260, vdim=20)],
     "mlstm_small_cap": [rec(gate_cap=1.5), rec(gate_cap=1.5)],
     "dense_ff": [attn(dense(ff=33), v_mix=False)],
     "experts_top_one": [attn(moe(top=1, count=1, keep=1))],

@@ -251,9 +251,14 @@ __global__ __launch_bounds__(256) void gqa_attn_merge_kernel(GqaAttnArgs a) {
 // ---- matrix memory (mLSTM).  Per head: a [dim][vdim] matrix S, a [dim] vector n and a running maximum mx (log scale), all fp32, all zero (mx too) at a
 // sequence's start.  For every token, with log gates i = cap tanh(zi / cap), f = logsigmoid(cap tanh(zf / cap)):
 //   mx' = max(f + mx, i);  S' = exp(f + mx - mx') S + exp(i - mx') k v^T;  n' likewise with k;  o = S'^T q / (max(|n' . q|, exp(-mx')) + 1e-6)
-// One workgroup per (entry, head, 64 value columns) walks the entry's tokens in order: lane = column, wave w holds rows [w DPER, (w + 1) DPER) of its
-// columns in registers.  n . q is computed by every workgroup of the head; n and mx are double-buffered per slot (buffer `par` is read, `par ^ 1`
-// written), because the workgroups of a head's other columns read them too.  The outputs leave un-normed (mlstm_out_kernel follows).
+// One workgroup per (entry, head, 64 value columns) walks the entry's tokens in order, MLSTM_TB at a time:
+//   stage   q (scaled), k, the workgroup's v columns and the gate pre-activations of the block's tokens into LDS (coalesced)
+//   gates   one thread per token: i, f, then mx' and the three factors exp(f + mx - mx'), exp(i - mx'), exp(-mx') from prefix sums over the block
+//           (mx'_t = B_t + max(mx_before, max_{s<=t} (i_s - B_s)), B_t = f_0 + .. + f_t: the recurrence unrolled)
+//   scan    no barrier inside: a wave owns 16 columns, its lanes = 4 row groups x 16 columns, each lane keeps DPER rows of its column in registers;
+//           S^T q is summed over the row groups with two lane exchanges, n . q (every wave computes it) with one wave sum
+// n and mx are double-buffered per slot (buffer `par` is read, `par ^ 1` written), because the workgroups of a head's other columns read them too.
+// The outputs leave un-normed (mlstm_out_kernel follows).
 struct MlstmArgs {
   const float* proj; long long ldp;     // [T][q | k | v | g | zi | zf]: q, k per head [dim]; v, g per head [vdim]; zi, zf per head (biases added)
   int heads, dim, vdim;
@@ -264,18 +269,19 @@ struct MlstmArgs {
   size_t n_buf, mx_buf;                 // elements between the two buffers
   float* hs; long long ldh;             // [T][heads * vdim]
 };
+constexpr int MLSTM_TB = 16;
 __device__ __forceinline__ float log_sigmoid(float z) { return fminf(z, 0.f) - log1pf(expf(-fabsf(z))); }
-template <int DPER>
+template <int DPER>      // rows per lane: 4 DPER >= dim
 __global__ __launch_bounds__(256) void mlstm_scan_kernel(StepMeta m, MlstmArgs a) {
-  constexpr int NPL = (DPER + 63) / 64;
-  __shared__ float s_o[2][4][64];
-  __shared__ float s_n[2][4];
-  const int e = blockIdx.x, h = blockIdx.y, lane = threadIdx.x & 63, wv = threadIdx.x >> 6;
-  const int j = blockIdx.z * 64 + lane;
+  constexpr int NPL = (DPER + 15) / 16, DP = 4 * DPER, TB = MLSTM_TB;
+  __shared__ __attribute__((aligned(16))) float s_q[TB][DP], s_k[TB][DP];
+  __shared__ float s_v[TB][64], s_zi[TB], s_zf[TB], s_keep[TB], s_take[TB], s_emn[TB], s_mx[2];
+  const int e = blockIdx.x, h = blockIdx.y, tid = threadIdx.x, lane = tid & 63, wv = tid >> 6, rg = lane >> 4, cl = lane & 15;
+  const int jl = wv * 16 + cl, j = blockIdx.z * 64 + jl;
   const int start = m.ent_start[e], cnt = m.ent_count[e], row = m.ent_row[e], par = m.ent_par[e];
   const bool fresh = m.tok_pos[start] == 0;
-  const int d0 = wv * DPER;
-  const int oq = h * a.dim, ok = a.heads * a.dim + h * a.dim, ov = 2 * a.heads * a.dim + h * a.vdim;
+  const int d0 = rg * DPER;
+  const int oq = h * a.dim, ok = a.heads * a.dim + h * a.dim, ov = 2 * a.heads * a.dim + h * a.vdim + blockIdx.z * 64;
   const int oi = 2 * a.heads * a.dim + 2 * a.heads * a.vdim + h, of = oi + a.heads;
   float* Sg = a.S + ((size_t)row * a.heads + h) * (size_t)a.dim * a.vdim;
   const float* n_old = a.n + (size_t)par * a.n_buf + ((size_t)row * a.heads + h) * a.dim;
@@ -284,48 +290,67 @@ __global__ __launch_bounds__(256) void mlstm_scan_kernel(StepMeta m, MlstmArgs a
 #pragma unroll
   for (int dd = 0; dd < DPER; dd++) { const int d = d0 + dd; S[dd] = (!fresh && d < a.dim && j < a.vdim) ? Sg[(size_t)d * a.vdim + j] : 0.f; }
 #pragma unroll
-  for (int k = 0; k < NPL; k++) { const int dl = lane + 64 * k, d = d0 + dl; nn[k] = (!fresh && dl < DPER && d < a.dim) ? n_old[d] : 0.f; }
-  float mx = fresh ? 0.f : a.mx[(size_t)par * a.mx_buf + (size_t)row * a.heads + h];
-  for (int i = 0; i < cnt; i++) {
-    const float* r = a.proj + (size_t)(start + i) * a.ldp;
-    const float ig = a.cap * tanhf(r[oi] / a.cap), fl = log_sigmoid(a.cap * tanhf(r[of] / a.cap));
-    const float mn = fmaxf(fl + mx, ig);
-    const float keep = expf(fl + mx - mn), take = expf(ig - mn);
-    const float vj = j < a.vdim ? r[ov + lane + blockIdx.z * 64] : 0.f;
-    const float tv = take * vj;
-    float po = 0.f;
+  for (int k = 0; k < NPL; k++) { const int dl = cl + 16 * k, d = d0 + dl; nn[k] = (!fresh && dl < DPER && d < a.dim) ? n_old[d] : 0.f; }
+  if (tid == 0) s_mx[0] = fresh ? 0.f : a.mx[(size_t)par * a.mx_buf + (size_t)row * a.heads + h];
+  for (int t0 = 0, blk = 0; t0 < cnt; t0 += TB, blk++) {
+    const int nb = min(TB, cnt - t0);
+    __syncthreads();                                       // the previous block's scan has read its rows
+    for (int i = tid; i < nb * DP; i += 256) {
+      const int t = i / DP, d = i - t * DP;
+      const float* r = a.proj + (size_t)(start + t0 + t) * a.ldp;
+      s_q[t][d] = d < a.dim ? r[oq + d] * a.qscale : 0.f;
+      s_k[t][d] = d < a.dim ? r[ok + d] : 0.f;
+    }
+    for (int i = tid; i < nb * 64; i += 256) {
+      const int t = i >> 6, c = i & 63;
+      s_v[t][c] = blockIdx.z * 64 + c < a.vdim ? a.proj[(size_t)(start + t0 + t) * a.ldp + ov + c] : 0.f;
+    }
+    if (tid < nb) {
+      const float* r = a.proj + (size_t)(start + t0 + tid) * a.ldp;
+      s_zi[tid] = a.cap * tanhf(r[oi] / a.cap);
+      s_zf[tid] = log_sigmoid(a.cap * tanhf(r[of] / a.cap));
+    }
+    __syncthreads();
+    if (tid < nb) {
+      const float mprev = s_mx[blk & 1];
+      float bs = 0.f, c = -INFINITY, mbefore = mprev;      // mbefore: the maximum after token tid - 1
+      for (int s2 = 0; s2 <= tid; s2++) {
+        if (s2 == tid) mbefore = s2 == 0 ? mprev : bs + fmaxf(mprev, c);
+        bs += s_zf[s2];
+        c = fmaxf(c, s_zi[s2] - bs);
+      }
+      const float mn = bs + fmaxf(mprev, c);
+      s_keep[tid] = expf(s_zf[tid] + mbefore - mn); s_take[tid] = expf(s_zi[tid] - mn); s_emn[tid] = expf(-mn);
+      if (tid == nb - 1) s_mx[(blk + 1) & 1] = mn;
+    }
+    __syncthreads();
+    for (int t = 0; t < nb; t++) {
+      const float keep = s_keep[t], tv = s_take[t] * s_v[t][jl];
+      float po = 0.f;
 #pragma unroll
-    for (int dd = 0; dd < DPER; dd++) {
-      const int d = min(d0 + dd, a.dim - 1);
-      const bool live = d0 + dd < a.dim;
-      const float kd = live ? r[ok + d] : 0.f, qd = live ? r[oq + d] * a.qscale : 0.f;
-      S[dd] = fmaf(keep, S[dd], kd * tv);
-      po = fmaf(S[dd], qd, po);
-    }
-    float pn = 0.f;
+      for (int dd = 0; dd < DPER; dd += 4) {
+        const f32x4 k4 = *reinterpret_cast<const f32x4*>(&s_k[t][d0 + dd]), q4 = *reinterpret_cast<const f32x4*>(&s_q[t][d0 + dd]);
 #pragma unroll
-    for (int k = 0; k < NPL; k++) {
-      const int dl = lane + 64 * k, d = d0 + dl;
-      if (dl < DPER && d < a.dim) { nn[k] = fmaf(keep, nn[k], take * r[ok + d]); pn = fmaf(nn[k], r[oq + d] * a.qscale, pn); }
+        for (int u = 0; u < 4; u++) { S[dd + u] = fmaf(keep, S[dd + u], k4[u] * tv); po = fmaf(S[dd + u], q4[u], po); }
+      }
+      float pn = 0.f;
+#pragma unroll
+      for (int k = 0; k < NPL; k++) {
+        const int dl = cl + 16 * k;
+        if (dl < DPER) { nn[k] = fmaf(keep, nn[k], s_take[t] * s_k[t][d0 + dl]); pn = fmaf(nn[k], s_q[t][d0 + dl], pn); }
+      }
+      po += __shfl_xor(po, 16, 64); po += __shfl_xor(po, 32, 64);
+      pn = wave_sum(pn);
+      if (rg == 0 && j < a.vdim) a.hs[(size_t)(start + t0 + t) * a.ldh + (size_t)h * a.vdim + j] = po / (fmaxf(fabsf(pn), s_emn[t]) + 1e-6f);
     }
-    pn = wave_sum(pn);
-    const int b = i & 1;
-    s_o[b][wv][lane] = po;
-    if (lane == 0) s_n[b][wv] = pn;
-    __syncthreads();      // one meeting per token: the buffers alternate, and no wave can run two tokens ahead of another
-    if (wv == 0 && j < a.vdim) {
-      const float o = (s_o[b][0][lane] + s_o[b][1][lane]) + (s_o[b][2][lane] + s_o[b][3][lane]);
-      const float nq = (s_n[b][0] + s_n[b][1]) + (s_n[b][2] + s_n[b][3]);
-      a.hs[(size_t)(start + i) * a.ldh + (size_t)h * a.vdim + j] = o / (fmaxf(fabsf(nq), expf(-mn)) + 1e-6f);
-    }
-    mx = mn;
   }
+  __syncthreads();
 #pragma unroll
   for (int dd = 0; dd < DPER; dd++) { const int d = d0 + dd; if (d < a.dim && j < a.vdim) Sg[(size_t)d * a.vdim + j] = S[dd]; }
-  if (blockIdx.z == 0) {
+  if (blockIdx.z == 0 && wv == 0) {
 #pragma unroll
-    for (int k = 0; k < NPL; k++) { const int dl = lane + 64 * k, d = d0 + dl; if (dl < DPER && d < a.dim) n_new[d] = nn[k]; }
-    if (threadIdx.x == 0) a.mx[(size_t)(par ^ 1) * a.mx_buf + (size_t)row * a.heads + h] = mx;
+    for (int k = 0; k < NPL; k++) { const int dl = cl + 16 * k, d = d0 + dl; if (dl < DPER && d < a.dim) n_new[d] = nn[k]; }
+    if (tid == 0) a.mx[(size_t)(par ^ 1) * a.mx_buf + (size_t)row * a.heads + h] = s_mx[((cnt + TB - 1) / TB) & 1];
   }
 }
 

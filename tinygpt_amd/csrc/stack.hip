@@ -411,8 +411,9 @@ int run_mlstm(tgx_ctx* c, const tgx::StepMeta& m, StackLayerW& w, const float* h
   ma.S = w.mS; ma.n = w.mn; ma.mx = w.mm; ma.n_buf = (size_t)sm->d.max_seqs * H * ld.dim; ma.mx_buf = (size_t)sm->d.max_seqs * H;
   ma.hs = sm->hs; ma.ldh = vd;
   const dim3 grid(S, H, (ld.vdim + 63) / 64);
-  const int dper = (ld.dim + 3) / 4;
-  if (dper <= 16) hipLaunchKernelGGL(tgx::mlstm_scan_kernel<16>, grid, dim3(256), 0, c->stream, m, ma);
+  const int dper = (ld.dim + 3) / 4;      // rows per lane: four row groups share a column
+  if (dper <= 8) hipLaunchKernelGGL(tgx::mlstm_scan_kernel<8>, grid, dim3(256), 0, c->stream, m, ma);
+  else if (dper <= 16) hipLaunchKernelGGL(tgx::mlstm_scan_kernel<16>, grid, dim3(256), 0, c->stream, m, ma);
   else if (dper <= 32) hipLaunchKernelGGL(tgx::mlstm_scan_kernel<32>, grid, dim3(256), 0, c->stream, m, ma);
   else if (dper <= 64) hipLaunchKernelGGL(tgx::mlstm_scan_kernel<64>, grid, dim3(256), 0, c->stream, m, ma);
   else hipLaunchKernelGGL(tgx::mlstm_scan_kernel<128>, grid, dim3(256), 0, c->stream, m, ma);
