@@ -445,3 +445,25 @@ def test_matrix_core_attention_equals_the_lane_kernel(heads, kv, dim, vdim):
     check(outs[0][[0, 1, 2, 4, 8, 9]], want, "bf16")               # a's positions 0, 1, 69, 130, 131, 199 in the order the steps returned them
     check(outs[0][[6, 7]], want_of(cfg, w, b)[[3, 74]], "bf16")
     fast.close(); slow.close()
+
+
+@pytest.mark.parametrize("dim,vdim", [(6, 8), (24, 70), (128, 40), (250, 33)])
+def test_both_column_splits_of_the_matrix_memory_scan(dim, vdim):
+    """the scan gives a wave sixteen columns, or eight when the step leaves most of the chip idle: the same steps through both (and against the oracle)"""
+    cfg = config([rec(dense(), heads=2, dim=dim, vdim=vdim), rec(heads=3, dim=dim, vdim=vdim)], width=32)
+    w = mo.random_tensors(cfg, dim)
+    tens = {k: np.asarray(v, np.float32) for k, v in w.items()}
+    a, b = tokens(cfg, 90, 1), tokens(cfg, 37, 2)
+    outs = []
+    for narrow in (0, 1):
+        eng = SlotEngine(desc=stack_desc_from_config(cfg, "fp32", max_seqs=4, max_ctx=256, budget_tokens=512), tensors=tens)
+        eng.model.set_option("mlstm.narrow", narrow)
+        o = [eng.step([("a", a[:50], [0, 31, 32, 49]), ("b", b[:1], [0])])]
+        o.append(eng.step([("a", a[50:52], [1]), ("b", b[1:36], [34])]))
+        o.append(eng.step([("a", a[52:], [37]), ("b", b[36:], [0])]))
+        outs.append(np.concatenate(o))
+        eng.close()
+    wa, wb = want_of(cfg, w, a), want_of(cfg, w, b)
+    want = np.stack([wa[0], wa[31], wa[32], wa[49], wb[0], wa[51], wb[35], wa[89], wb[36]])
+    check(outs[0], want, "fp32", "sixteen columns")
+    check(outs[1], want, "fp32", "eight columns")

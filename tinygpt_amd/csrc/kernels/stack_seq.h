@@ -251,12 +251,14 @@ __global__ __launch_bounds__(256) void gqa_attn_merge_kernel(GqaAttnArgs a) {
 // ---- matrix memory (mLSTM).  Per head: a [dim][vdim] matrix S, a [dim] vector n and a running maximum mx (log scale), all fp32, all zero (mx too) at a
 // sequence's start.  For every token, with log gates i = cap tanh(zi / cap), f = logsigmoid(cap tanh(zf / cap)):
 //   mx' = max(f + mx, i);  S' = exp(f + mx - mx') S + exp(i - mx') k v^T;  n' likewise with k;  o = S'^T q / (max(|n' . q|, exp(-mx')) + 1e-6)
-// One workgroup per (entry, head, 64 value columns) walks the entry's tokens in order, MLSTM_TB at a time:
+// One workgroup per (entry, head, 4 CW value columns; CW = 16, or 8 when the step has few entries and heads) walks the entry's tokens in order, a block of
+// 8 .. 32 at a time:
 //   stage   q (scaled), k, the workgroup's v columns and the gate pre-activations of the block's tokens into LDS (coalesced)
 //   gates   one thread per token: i, f, then mx' and the three factors exp(f + mx - mx'), exp(i - mx'), exp(-mx') from prefix sums over the block
 //           (mx'_t = B_t + max(mx_before, max_{s<=t} (i_s - B_s)), B_t = f_0 + .. + f_t: the recurrence unrolled)
-//   scan    no barrier inside: a wave owns 16 columns, its lanes = 4 row groups x 16 columns, each lane keeps DPER rows of its column in registers;
-//           S^T q is summed over the row groups with two lane exchanges, n . q (every wave computes it) with one wave sum
+//   scan    no barrier and no lane exchange inside: a wave owns CW columns, its lanes = 64 / CW row groups x CW columns, each lane keeps DPER rows of its
+//           column in registers and leaves its partial sums of S^T q and n . q (every wave computes the latter) per token in LDS
+//   out     the partial sums of the block's tokens are added up (over the row groups; over the wave for n . q) and divided
 // n and mx are double-buffered per slot (buffer `par` is read, `par ^ 1` written), because the workgroups of a head's other columns read them too.
 // The outputs leave un-normed (mlstm_out_kernel follows).
 struct MlstmArgs {
@@ -269,19 +271,21 @@ struct MlstmArgs {
   size_t n_buf, mx_buf;                 // elements between the two buffers
   float* hs; long long ldh;             // [T][heads * vdim]
 };
-constexpr int MLSTM_TB = 16;
 __device__ __forceinline__ float log_sigmoid(float z) { return fminf(z, 0.f) - log1pf(expf(-fabsf(z))); }
-template <int DPER>      // rows per lane: 4 DPER >= dim
+template <int DPER, int CW>      // rows per lane and columns per wave: (64 / CW) DPER >= dim
 __global__ __launch_bounds__(256) void mlstm_scan_kernel(StepMeta m, MlstmArgs a) {
-  constexpr int NPL = (DPER + 15) / 16, DP = 4 * DPER, TB = MLSTM_TB;
-  __shared__ __attribute__((aligned(16))) float s_q[TB][DP], s_k[TB][DP];
-  __shared__ float s_v[TB][64], s_zi[TB], s_zf[TB], s_keep[TB], s_take[TB], s_emn[TB], s_mx[2];
-  const int e = blockIdx.x, h = blockIdx.y, tid = threadIdx.x, lane = tid & 63, wv = tid >> 6, rg = lane >> 4, cl = lane & 15;
-  const int jl = wv * 16 + cl, j = blockIdx.z * 64 + jl;
+  constexpr int RG = 64 / CW, NPL = (DPER + CW - 1) / CW, DP = RG * DPER, LP = DPER + 4, CB = 4 * CW;      // LP: a row group's LDS stride (the groups' reads fall into different banks)
+  constexpr int TB = DP <= 128 ? 32 : (DP <= 256 ? 16 : 8);                                             // tokens per block: 32 KB of staged q and k
+  constexpr int NQ = TB * DP / 256, NV = (TB * CB + 255) / 256;
+  __shared__ __attribute__((aligned(16))) float s_q[TB][RG * LP], s_k[TB][RG * LP];
+  __shared__ float s_v[TB][CB], s_zi[TB], s_zf[TB], s_keep[TB], s_take[TB], s_emn[TB], s_mx[2];
+  __shared__ float s_po[TB][4][64], s_pn[TB][4][64];
+  const int e = blockIdx.x, h = blockIdx.y, tid = threadIdx.x, lane = tid & 63, wv = tid >> 6, rg = lane / CW, cl = lane % CW;
+  const int jl = wv * CW + cl, j = blockIdx.z * CB + jl;
   const int start = m.ent_start[e], cnt = m.ent_count[e], row = m.ent_row[e], par = m.ent_par[e];
   const bool fresh = m.tok_pos[start] == 0;
-  const int d0 = rg * DPER;
-  const int oq = h * a.dim, ok = a.heads * a.dim + h * a.dim, ov = 2 * a.heads * a.dim + h * a.vdim + blockIdx.z * 64;
+  const int d0 = rg * DPER, l0 = rg * LP;
+  const int oq = h * a.dim, ok = a.heads * a.dim + h * a.dim, ov = 2 * a.heads * a.dim + h * a.vdim + blockIdx.z * CB;
   const int oi = 2 * a.heads * a.dim + 2 * a.heads * a.vdim + h, of = oi + a.heads;
   float* Sg = a.S + ((size_t)row * a.heads + h) * (size_t)a.dim * a.vdim;
   const float* n_old = a.n + (size_t)par * a.n_buf + ((size_t)row * a.heads + h) * a.dim;
@@ -290,27 +294,40 @@ __global__ __launch_bounds__(256) void mlstm_scan_kernel(StepMeta m, MlstmArgs a
 #pragma unroll
   for (int dd = 0; dd < DPER; dd++) { const int d = d0 + dd; S[dd] = (!fresh && d < a.dim && j < a.vdim) ? Sg[(size_t)d * a.vdim + j] : 0.f; }
 #pragma unroll
-  for (int k = 0; k < NPL; k++) { const int dl = cl + 16 * k, d = d0 + dl; nn[k] = (!fresh && dl < DPER && d < a.dim) ? n_old[d] : 0.f; }
+  for (int k = 0; k < NPL; k++) { const int dl = cl + CW * k, d = d0 + dl; nn[k] = (!fresh && dl < DPER && d < a.dim) ? n_old[d] : 0.f; }
   if (tid == 0) s_mx[0] = fresh ? 0.f : a.mx[(size_t)par * a.mx_buf + (size_t)row * a.heads + h];
+  // the next block's inputs travel in registers while the current block is scanned
+  float rq[NQ], rk[NQ], rv[NV], rzi = 0.f, rzf = 0.f;
+  auto fetch = [&](int t0) {
+    const int nb = min(TB, cnt - t0);
+#pragma unroll
+    for (int u = 0; u < NQ; u++) {
+      const int i = tid + 256 * u, t = i / DP, d = i - t * DP;
+      const bool on = t < nb && d < a.dim;
+      const float* r = a.proj + (size_t)(start + t0 + min(t, nb - 1)) * a.ldp;
+      rq[u] = on ? r[oq + d] : 0.f; rk[u] = on ? r[ok + d] : 0.f;
+    }
+#pragma unroll
+    for (int u = 0; u < NV; u++) {
+      const int i = tid + 256 * u, t = i / CB, c = i - t * CB;
+      rv[u] = (t < nb && blockIdx.z * CB + c < a.vdim) ? a.proj[(size_t)(start + t0 + t) * a.ldp + ov + c] : 0.f;
+    }
+    if (tid < nb) { const float* r = a.proj + (size_t)(start + t0 + tid) * a.ldp; rzi = r[oi]; rzf = r[of]; }
+  };
+  fetch(0);
   for (int t0 = 0, blk = 0; t0 < cnt; t0 += TB, blk++) {
     const int nb = min(TB, cnt - t0);
-    __syncthreads();                                       // the previous block's scan has read its rows
-    for (int i = tid; i < nb * DP; i += 256) {
-      const int t = i / DP, d = i - t * DP;
-      const float* r = a.proj + (size_t)(start + t0 + t) * a.ldp;
-      s_q[t][d] = d < a.dim ? r[oq + d] * a.qscale : 0.f;
-      s_k[t][d] = d < a.dim ? r[ok + d] : 0.f;
+    __syncthreads();                                       // the previous block's rows and partial sums have been read
+#pragma unroll
+    for (int u = 0; u < NQ; u++) {
+      const int i = tid + 256 * u, t = i / DP, d = i - t * DP, at = (d / DPER) * LP + d % DPER;
+      s_q[t][at] = rq[u] * a.qscale; s_k[t][at] = rk[u];
     }
-    for (int i = tid; i < nb * 64; i += 256) {
-      const int t = i >> 6, c = i & 63;
-      s_v[t][c] = blockIdx.z * 64 + c < a.vdim ? a.proj[(size_t)(start + t0 + t) * a.ldp + ov + c] : 0.f;
-    }
-    if (tid < nb) {
-      const float* r = a.proj + (size_t)(start + t0 + tid) * a.ldp;
-      s_zi[tid] = a.cap * tanhf(r[oi] / a.cap);
-      s_zf[tid] = log_sigmoid(a.cap * tanhf(r[of] / a.cap));
-    }
+#pragma unroll
+    for (int u = 0; u < NV; u++) { const int i = tid + 256 * u; if (i < TB * CB) s_v[i / CB][i % CB] = rv[u]; }
+    if (tid < nb) { s_zi[tid] = a.cap * tanhf(rzi / a.cap); s_zf[tid] = log_sigmoid(a.cap * tanhf(rzf / a.cap)); }
     __syncthreads();
+    if (t0 + TB < cnt) fetch(t0 + TB);
     if (tid < nb) {
       const float mprev = s_mx[blk & 1];
       float bs = 0.f, c = -INFINITY, mbefore = mprev;      // mbefore: the maximum after token tid - 1
@@ -329,19 +346,28 @@ __global__ __launch_bounds__(256) void mlstm_scan_kernel(StepMeta m, MlstmArgs a
       float po = 0.f;
 #pragma unroll
       for (int dd = 0; dd < DPER; dd += 4) {
-        const f32x4 k4 = *reinterpret_cast<const f32x4*>(&s_k[t][d0 + dd]), q4 = *reinterpret_cast<const f32x4*>(&s_q[t][d0 + dd]);
+        const f32x4 k4 = *reinterpret_cast<const f32x4*>(&s_k[t][l0 + dd]), q4 = *reinterpret_cast<const f32x4*>(&s_q[t][l0 + dd]);
 #pragma unroll
         for (int u = 0; u < 4; u++) { S[dd + u] = fmaf(keep, S[dd + u], k4[u] * tv); po = fmaf(S[dd + u], q4[u], po); }
       }
       float pn = 0.f;
 #pragma unroll
       for (int k = 0; k < NPL; k++) {
-        const int dl = cl + 16 * k;
-        if (dl < DPER) { nn[k] = fmaf(keep, nn[k], s_take[t] * s_k[t][d0 + dl]); pn = fmaf(nn[k], s_q[t][d0 + dl], pn); }
+        const int dl = cl + CW * k;
+        if (dl < DPER) { nn[k] = fmaf(keep, nn[k], s_take[t] * s_k[t][l0 + dl]); pn = fmaf(nn[k], s_q[t][l0 + dl], pn); }
       }
-      po += __shfl_xor(po, 16, 64); po += __shfl_xor(po, 32, 64);
-      pn = wave_sum(pn);
-      if (rg == 0 && j < a.vdim) a.hs[(size_t)(start + t0 + t) * a.ldh + (size_t)h * a.vdim + j] = po / (fmaxf(fabsf(pn), s_emn[t]) + 1e-6f);
+      s_po[t][wv][lane] = po; s_pn[t][wv][lane] = pn;      // partial sums over this lane's rows: reduced after the block, off the recurrence's critical path
+    }
+    __syncthreads();
+    // the block's outputs: row group rg of a wave takes tokens rg, rg + RG, ...; its CW lanes are the wave's columns
+    for (int t = rg; t < nb; t += RG) {
+      float o = 0.f, nq = 0.f;
+#pragma unroll
+      for (int g = 0; g < RG; g++) o += s_po[t][wv][g * CW + cl];
+#pragma unroll
+      for (int g = 0; g < RG; g++) nq += s_pn[t][wv][RG * cl + g];
+      nq = row_group_sum<CW>(nq);
+      if (j < a.vdim) a.hs[(size_t)(start + t0 + t) * a.ldh + (size_t)h * a.vdim + j] = o / (fmaxf(fabsf(nq), s_emn[t]) + 1e-6f);
     }
   }
   __syncthreads();
@@ -349,7 +375,7 @@ __global__ __launch_bounds__(256) void mlstm_scan_kernel(StepMeta m, MlstmArgs a
   for (int dd = 0; dd < DPER; dd++) { const int d = d0 + dd; if (d < a.dim && j < a.vdim) Sg[(size_t)d * a.vdim + j] = S[dd]; }
   if (blockIdx.z == 0 && wv == 0) {
 #pragma unroll
-    for (int k = 0; k < NPL; k++) { const int dl = cl + 16 * k, d = d0 + dl; if (dl < DPER && d < a.dim) n_new[d] = nn[k]; }
+    for (int k = 0; k < NPL; k++) { const int dl = cl + CW * k, d = d0 + dl; if (dl < DPER && d < a.dim) n_new[d] = nn[k]; }
     if (tid == 0) a.mx[(size_t)(par ^ 1) * a.mx_buf + (size_t)row * a.heads + h] = s_mx[((cnt + TB - 1) / TB) & 1];
   }
 }

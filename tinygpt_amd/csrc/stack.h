@@ -72,6 +72,7 @@ struct StackModel {
   int attn_split_min_keys = 2048;      // option attn.split_min: steps of few tokens split a sequence's keys between workgroups from this context on
   int attn_mfma = 1;                   // option attn.mfma: 0 keeps every layer on the lane-per-channel attention kernels
   int gemv = 1;                        // option stack.gemv: 0 sends products of few rows through the matrix-core tiles as well
+  int mlstm_narrow = -1;               // option mlstm.narrow: the matrix-memory scan's columns per wave (1: eight, 0: sixteen, -1: by the step's entries and heads)
   int gemm_wt = 0;                     // option stack.gemm_wt: force the product's tile (1: 64 x 64, 2: 128 x 128); 0 = by the number of tiles
 };
 

@@ -410,13 +410,23 @@ int run_mlstm(tgx_ctx* c, const tgx::StepMeta& m, StackLayerW& w, const float* h
   ma.proj = sm->proj; ma.ldp = nin; ma.heads = H; ma.dim = ld.dim; ma.vdim = ld.vdim; ma.cap = ld.gate_cap; ma.qscale = 1.0f / sqrtf((float)ld.dim);
   ma.S = w.mS; ma.n = w.mn; ma.mx = w.mm; ma.n_buf = (size_t)sm->d.max_seqs * H * ld.dim; ma.mx_buf = (size_t)sm->d.max_seqs * H;
   ma.hs = sm->hs; ma.ldh = vd;
-  const dim3 grid(S, H, (ld.vdim + 63) / 64);
-  const int dper = (ld.dim + 3) / 4;      // rows per lane: four row groups share a column
-  if (dper <= 8) hipLaunchKernelGGL(tgx::mlstm_scan_kernel<8>, grid, dim3(256), 0, c->stream, m, ma);
-  else if (dper <= 16) hipLaunchKernelGGL(tgx::mlstm_scan_kernel<16>, grid, dim3(256), 0, c->stream, m, ma);
-  else if (dper <= 32) hipLaunchKernelGGL(tgx::mlstm_scan_kernel<32>, grid, dim3(256), 0, c->stream, m, ma);
-  else if (dper <= 64) hipLaunchKernelGGL(tgx::mlstm_scan_kernel<64>, grid, dim3(256), 0, c->stream, m, ma);
-  else hipLaunchKernelGGL(tgx::mlstm_scan_kernel<128>, grid, dim3(256), 0, c->stream, m, ma);
+  // columns per wave: 16, or 8 (twice the workgroups, half the rows per lane) while the step's entries and heads leave most of the chip idle
+  const bool narrow = ld.dim <= 256 && (sm->mlstm_narrow >= 0 ? sm->mlstm_narrow != 0 : (long long)S * H * ((ld.vdim + 63) / 64) * 2 <= c->num_cus);
+  if (narrow) {
+    const dim3 grid(S, H, (ld.vdim + 31) / 32);
+    const int dper = (ld.dim + 7) / 8;
+    if (dper <= 8) hipLaunchKernelGGL((tgx::mlstm_scan_kernel<8, 8>), grid, dim3(256), 0, c->stream, m, ma);
+    else if (dper <= 16) hipLaunchKernelGGL((tgx::mlstm_scan_kernel<16, 8>), grid, dim3(256), 0, c->stream, m, ma);
+    else hipLaunchKernelGGL((tgx::mlstm_scan_kernel<32, 8>), grid, dim3(256), 0, c->stream, m, ma);
+  } else {
+    const dim3 grid(S, H, (ld.vdim + 63) / 64);
+    const int dper = (ld.dim + 3) / 4;      // rows per lane: four row groups share a column
+    if (dper <= 8) hipLaunchKernelGGL((tgx::mlstm_scan_kernel<8, 16>), grid, dim3(256), 0, c->stream, m, ma);
+    else if (dper <= 16) hipLaunchKernelGGL((tgx::mlstm_scan_kernel<16, 16>), grid, dim3(256), 0, c->stream, m, ma);
+    else if (dper <= 32) hipLaunchKernelGGL((tgx::mlstm_scan_kernel<32, 16>), grid, dim3(256), 0, c->stream, m, ma);
+    else if (dper <= 64) hipLaunchKernelGGL((tgx::mlstm_scan_kernel<64, 16>), grid, dim3(256), 0, c->stream, m, ma);
+    else hipLaunchKernelGGL((tgx::mlstm_scan_kernel<128, 16>), grid, dim3(256), 0, c->stream, m, ma);
+  }
   tgx::MlstmOutArgs oa{};
   oa.hs = sm->hs; oa.ldh = vd; oa.w = w.head_w; oa.gate = sm->proj + 2 * qd + vd; oa.ldg = nin; oa.out = sm->o; oa.ldo = vd; oa.vdim = ld.vdim; oa.eps = sm->d.norm_eps;
   hipLaunchKernelGGL(tgx::mlstm_out_kernel, dim3(T, H), dim3(64), 0, c->stream, oa);
