@@ -327,7 +327,7 @@ def modepel_desc(key, z, L, V, dtype, B, ctx):
         if i == 0:
             l.mlp, l.ff = "dense", z["top"] * z["ff"]
         else:
-            l.mlp, l.experts, l.identity, l.top, l.ff, l.groups, l.groups_keep, l.router_scale, l.shared_ff = "moe", z["experts"], z["experts"] // 4, z["top"], z["ff"], 4, 2, 1.5, z["ff"]
+            l.mlp, l.experts, l.identity, l.top, l.ff, l.groups, l.groups_keep, l.router_scale, l.shared_ff = "moe", z["experts"], 4, z["top"], z["ff"], 4, 2, 1.5, z["ff"]
         layers.append(l)
     return StackDesc(family="modepel", width=W, vocab=V, compute_dtype=dtype, max_seqs=B, max_ctx=ctx, budget_tokens=B * (ctx + 64), norm_eps=1e-5, name=f"modepel-{key}", layers=layers)
 

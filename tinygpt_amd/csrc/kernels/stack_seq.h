@@ -275,7 +275,9 @@ __device__ __forceinline__ float log_sigmoid(float z) { return fminf(z, 0.f) - l
 template <int DPER, int CW>      // rows per lane and columns per wave: (64 / CW) DPER >= dim
 __global__ __launch_bounds__(256) void mlstm_scan_kernel(StepMeta m, MlstmArgs a) {
   constexpr int RG = 64 / CW, NPL = (DPER + CW - 1) / CW, DP = RG * DPER, LP = DPER + 4, CB = 4 * CW;      // LP: a row group's LDS stride (the groups' reads fall into different banks)
-  constexpr int TB = DP <= 128 ? 32 : (DP <= 256 ? 16 : 8);                                             // tokens per block: 32 KB of staged q and k
+  // tokens per block: the eight-column form runs alone on its compute unit (few workgroups) and takes long blocks; the sixteen-column form keeps its
+  // LDS (staged q and k, the partial sums) near 50 KB so that several workgroups share a compute unit
+  constexpr int TB = CW == 8 ? (DP <= 128 ? 32 : 16) : (DP <= 256 ? 16 : 8);
   constexpr int NQ = TB * DP / 256, NV = (TB * CB + 255) / 256;
   __shared__ __attribute__((aligned(16))) float s_q[TB][RG * LP], s_k[TB][RG * LP];
   __shared__ float s_v[TB][CB], s_zi[TB], s_zf[TB], s_keep[TB], s_take[TB], s_emn[TB], s_mx[2];
