@@ -3,13 +3,13 @@
 //
 // The query heads of one key / value head read the same cached rows, so a workgroup owns 32 ROWS = consecutive (token, query head of the group) pairs of
 // one entry of the step and one key / value head — eight tokens x four heads of a prompt portion, or the group's heads of one decoded token — and walks the
-// keys its rows see in tiles of 32 (the scheme of latent_attn_mfma_kernel, with separate key and value operands):
-//   1. S = Q K^T: the four waves split the head's dim channels (the contraction), each leaves a partial 32 x 32 tile in LDS
+// keys its rows see in tiles of 64 (the scheme of latent_attn_mfma_kernel, with separate key and value operands and two of its key tiles per barrier pair):
+//   1. S = Q K^T: the four waves split the head's dim channels (the contraction), each leaves a partial 32 x 64 tile in LDS
 //   2. softmax bookkeeping in fp32, eight rows per wave: sum of the partials, causal mask per row, running maximum / denominator (the denominator
 //      starts at exp(sink) where the design has a sink: a term without key or value), P as two 16-bit terms and the rows' rescale factors back to LDS
 //   3. O += P V: every wave owns 32 NT of the vdim output columns; its B operand comes from a TRANSPOSED copy of the value page ([channel][token]: eight
 //      consecutive keys of a channel are one 16-byte load) that the append kernel writes
-// Q (score scale folded in) enters as two 16-bit terms (one with option act.round16).  Key tiles never straddle a page (pages hold a multiple of 32
+// Q (score scale folded in) enters as two 16-bit terms (one with option act.round16).  Key tiles never straddle a page (pages hold a multiple of 64
 // tokens).  The output is multiplied by sigmoid(gate) where a gate is given.  SPLIT: blockIdx.z takes a range of the keys and leaves (m, l, O) records
 // for gqa_attn_merge_kernel.
 #pragma once
@@ -24,7 +24,7 @@ struct GqaMfmaArgs {
   const void* poolVT;                  // [pages][kv_heads * vdim][page]
   const float* gate; long long ldg;    // gate pre-activation of (t, h, c) at gate + t * ldg + h * vdim + c (nullptr: none)
   float* out; long long ldo;           // [T][heads * vdim]
-  float* part; int nsplit, keys_per;   // keys_per: a multiple of 32
+  float* part; int nsplit, keys_per;   // keys_per: a multiple of 64
   int heads, kv_heads, dim, vdim, terms;
   float scale, sink; int has_sink;
 };
@@ -32,8 +32,8 @@ struct GqaMfmaArgs {
 template <int DT, int ND, int NT, bool SPLIT>      // ND = dim / 64: 16-channel steps of a wave's share of the contraction; NT = ceil(vdim / 128): 32-column output tiles per wave
 __global__ __launch_bounds__(256) void gqa_attn_mfma_kernel(StepMeta m, GqaMfmaArgs a) {
   constexpr int RQ = 16 * ND, KS = ND;
-  __shared__ float s_part[4][32][33];
-  __shared__ __attribute__((aligned(16))) bf16_t s_ph[32][40], s_pl[32][40];
+  __shared__ float s_part[4][32][65];
+  __shared__ __attribute__((aligned(16))) bf16_t s_ph[32][72], s_pl[32][72];
   __shared__ float s_corr[32], s_l[32];
   const int e = blockIdx.y / a.kv_heads, kvh = blockIdx.y - e * a.kv_heads, Gq = a.heads / a.kv_heads;
   const int cnt = m.ent_count[e], start = m.ent_start[e], slot = m.ent_row[e];
@@ -71,8 +71,8 @@ __global__ __launch_bounds__(256) void gqa_attn_mfma_kernel(StepMeta m, GqaMfmaA
 #pragma unroll
     for (int r = 0; r < 16; r++) acc[t][r] = 0.f;
 
-  // softmax bookkeeping: wave wv keeps rows 8 wv .. 8 wv + 7, eight lanes a row, four keys a lane
-  const int srow = 8 * wv + (lane >> 3), kq = 4 * (lane & 7);
+  // softmax bookkeeping: wave wv keeps rows 8 wv .. 8 wv + 7, eight lanes a row, eight keys a lane
+  const int srow = 8 * wv + (lane >> 3), kq = 8 * (lane & 7);
   const int sr = r0 + srow;
   const bool svalid = sr < nrows;
   const int skeys = svalid ? past + sr / Gq + 1 : 0;
@@ -83,45 +83,51 @@ __global__ __launch_bounds__(256) void gqa_attn_mfma_kernel(StepMeta m, GqaMfmaA
     const size_t pg = (size_t)m.tbl[(size_t)slot * m.tbl_stride + (kt >> m.page_shift)];
     return poolK + ((pg << m.page_shift) + (kt & (page - 1)) + l31) * (size_t)kd + wv * RQ + 8 * half;
   };
-  u32x4 bq[KS];
+  u32x4 bq[2][KS];
   if (k0 < k1) {
     const bf16_t* cp = key_rows(k0);
 #pragma unroll
-    for (int kk = 0; kk < KS; kk++) bq[kk] = *reinterpret_cast<const u32x4*>(cp + 16 * kk);
+    for (int kk = 0; kk < KS; kk++) { bq[0][kk] = *reinterpret_cast<const u32x4*>(cp + 16 * kk); bq[1][kk] = *reinterpret_cast<const u32x4*>(cp + 32 * (size_t)kd + 16 * kk); }
   }
-  for (int kt = k0; kt < k1; kt += 32) {
+  for (int kt = k0; kt < k1; kt += 64) {
     const size_t pg = (size_t)m.tbl[(size_t)slot * m.tbl_stride + (kt >> m.page_shift)];
     const int off = kt & (page - 1);
-    u32x4 bt[NT][2];
+    u32x4 bt[NT][4];
 #pragma unroll
     for (int t = 0; t < NT; t++) {
       const int col = min(wv * 32 * NT + 32 * t + l31, a.vdim - 1);
       const bf16_t* tp = poolVT + ((pg * vd + (size_t)(kvh * a.vdim + col)) << m.page_shift) + off + 8 * half;
-      bt[t][0] = *reinterpret_cast<const u32x4*>(tp); bt[t][1] = *reinterpret_cast<const u32x4*>(tp + 16);
+#pragma unroll
+      for (int kk = 0; kk < 4; kk++) bt[t][kk] = *reinterpret_cast<const u32x4*>(tp + 16 * kk);
     }
-    // 1. partial scores over this wave's channels
-    f32x16 s;
+    // 1. partial scores over this wave's channels, keys kt .. kt + 31 and kt + 32 .. kt + 63
+    f32x16 s[2];
 #pragma unroll
-    for (int r = 0; r < 16; r++) s[r] = 0.f;
+    for (int h2 = 0; h2 < 2; h2++) {
 #pragma unroll
-    for (int kk = 0; kk < KS; kk++) {
-      const bf16x8 b = __builtin_bit_cast(bf16x8, bq[kk]);
-      s = mfma16<DT>(qh[kk], b, s);
-      if (a.terms > 1) s = mfma16<DT>(ql[kk], b, s);
+      for (int r = 0; r < 16; r++) s[h2][r] = 0.f;
+#pragma unroll
+      for (int kk = 0; kk < KS; kk++) {
+        const bf16x8 b = __builtin_bit_cast(bf16x8, bq[h2][kk]);
+        s[h2] = mfma16<DT>(qh[kk], b, s[h2]);
+        if (a.terms > 1) s[h2] = mfma16<DT>(ql[kk], b, s[h2]);
+      }
     }
-    if (kt + 32 < k1) {
-      const bf16_t* cp = key_rows(kt + 32);
+    if (kt + 64 < k1) {
+      const bf16_t* cp = key_rows(kt + 64);
 #pragma unroll
-      for (int kk = 0; kk < KS; kk++) bq[kk] = *reinterpret_cast<const u32x4*>(cp + 16 * kk);
+      for (int kk = 0; kk < KS; kk++) { bq[0][kk] = *reinterpret_cast<const u32x4*>(cp + 16 * kk); bq[1][kk] = *reinterpret_cast<const u32x4*>(cp + 32 * (size_t)kd + 16 * kk); }
     }
 #pragma unroll
-    for (int r = 0; r < 16; r++) s_part[wv][(r & 3) + 8 * (r >> 2) + 4 * half][l31] = s[r];
+    for (int h2 = 0; h2 < 2; h2++)
+#pragma unroll
+      for (int r = 0; r < 16; r++) s_part[wv][(r & 3) + 8 * (r >> 2) + 4 * half][32 * h2 + l31] = s[h2][r];
     __syncthreads();
     // 2. the rows' softmax state
     {
-      float sv[4], tmax = -INFINITY;
+      float sv[8], tmax = -INFINITY;
 #pragma unroll
-      for (int c = 0; c < 4; c++) {
+      for (int c = 0; c < 8; c++) {
         const float v = s_part[0][srow][kq + c] + s_part[1][srow][kq + c] + s_part[2][srow][kq + c] + s_part[3][srow][kq + c];
         sv[c] = (kt + kq + c < min(skeys, k1)) ? v : -INFINITY;
         tmax = fmaxf(tmax, sv[c]);
@@ -131,14 +137,17 @@ __global__ __launch_bounds__(256) void gqa_attn_mfma_kernel(StepMeta m, GqaMfmaA
       const bool dead = mn == -INFINITY;                  // nothing seen yet (a row of another split, or a padding row)
       const float corr = dead ? 1.f : expf(m_s - mn);
       float psum = 0.f;
-      bf16_t ph[4], pl[4];
+      bf16_t ph[8], pl[8];
 #pragma unroll
-      for (int c = 0; c < 4; c++) { const float p = dead ? 0.f : expf(sv[c] - mn); psum += p; split16<DT>(p, ph[c], pl[c]); }
+      for (int c = 0; c < 8; c++) { const float p = dead ? 0.f : expf(sv[c] - mn); psum += p; split16<DT>(p, ph[c], pl[c]); }
       psum += __shfl_xor(psum, 1, 64); psum += __shfl_xor(psum, 2, 64); psum += __shfl_xor(psum, 4, 64);
       l_s = fmaf(l_s, corr, psum);
       m_s = mn;
-      *reinterpret_cast<u32x2*>(&s_ph[srow][kq]) = u32x2{(unsigned int)ph[0] | ((unsigned int)ph[1] << 16), (unsigned int)ph[2] | ((unsigned int)ph[3] << 16)};
-      *reinterpret_cast<u32x2*>(&s_pl[srow][kq]) = u32x2{(unsigned int)pl[0] | ((unsigned int)pl[1] << 16), (unsigned int)pl[2] | ((unsigned int)pl[3] << 16)};
+      u32x4 uh, ul;
+#pragma unroll
+      for (int i = 0; i < 4; i++) { uh[i] = (unsigned int)ph[2 * i] | ((unsigned int)ph[2 * i + 1] << 16); ul[i] = (unsigned int)pl[2 * i] | ((unsigned int)pl[2 * i + 1] << 16); }
+      *reinterpret_cast<u32x4*>(&s_ph[srow][kq]) = uh;
+      *reinterpret_cast<u32x4*>(&s_pl[srow][kq]) = ul;
       if ((lane & 7) == 0) s_corr[srow] = corr;
     }
     __syncthreads();
@@ -146,9 +155,9 @@ __global__ __launch_bounds__(256) void gqa_attn_mfma_kernel(StepMeta m, GqaMfmaA
     float cr[16];
 #pragma unroll
     for (int r = 0; r < 16; r++) cr[r] = s_corr[(r & 3) + 8 * (r >> 2) + 4 * half];
-    bf16x8 pa[2], pb[2];
+    bf16x8 pa[4], pb[4];
 #pragma unroll
-    for (int kk = 0; kk < 2; kk++) {
+    for (int kk = 0; kk < 4; kk++) {
       pa[kk] = *reinterpret_cast<const bf16x8*>(&s_ph[l31][16 * kk + 8 * half]);
       pb[kk] = *reinterpret_cast<const bf16x8*>(&s_pl[l31][16 * kk + 8 * half]);
     }
@@ -158,7 +167,7 @@ __global__ __launch_bounds__(256) void gqa_attn_mfma_kernel(StepMeta m, GqaMfmaA
 #pragma unroll
       for (int r = 0; r < 16; r++) acc[t][r] *= cr[r];
 #pragma unroll
-      for (int kk = 0; kk < 2; kk++) {
+      for (int kk = 0; kk < 4; kk++) {
         const bf16x8 b = __builtin_bit_cast(bf16x8, bt[t][kk]);
         acc[t] = mfma16<DT>(pa[kk], b, acc[t]);
         if (a.terms > 1) acc[t] = mfma16<DT>(pb[kk], b, acc[t]);

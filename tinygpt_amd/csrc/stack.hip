@@ -355,7 +355,7 @@ int run_attention(tgx_ctx* c, const tgx::StepMeta& m, StackLayerW& w, const floa
     int nsplit = 1;
     if (max_keys >= sm->attn_split_min_keys && wgs < c->num_cus) {
       nsplit = (int)std::min<long long>(64, (2LL * c->num_cus) / wgs);
-      const int per = std::max(64, ((max_keys + nsplit - 1) / nsplit + 31) / 32 * 32);      // two key tiles per workgroup at least
+      const int per = std::max(64, ((max_keys + nsplit - 1) / nsplit + 63) / 64 * 64);      // whole key tiles
       nsplit = (max_keys + per - 1) / per;
       ma.keys_per = per;
     }
@@ -603,8 +603,8 @@ int create_sandwich_layers(tgx_ctx* c, const tgx_layer_desc* layers) {
       if (l.v_mix) {
         if ((rc = dev_alloc(c, &w.vmix, 1))) return rc;
         HIP_OK(c, hipMemset(w.vmix, 0, 4));
-        sm->missing.insert(p + "mix.vmix");
         w.vmode = mixing ? 2 : 1;
+        if (w.vmode == 2) sm->missing.insert(p + "mix.vmix");      // (the first mixing layer's number is never read: taken if the checkpoint has it, not asked for)
         mixing = true;
       }
       if (l.rot_dims > 0) {

@@ -21,7 +21,7 @@ void launch_nd(tgx_ctx* c, const tgx::StepMeta& m, const tgx::GqaMfmaArgs& a, di
 }  // namespace
 
 bool gqa_mfma_shapes_ok(int dt, int dim, int vdim, int page_shift, long long ldq) {
-  return dt != tgx::DT_F32 && (dim == 64 || dim == 128 || dim == 256) && vdim % 32 == 0 && vdim >= 32 && vdim <= 256 && page_shift >= 5 && ldq % 4 == 0;
+  return dt != tgx::DT_F32 && (dim == 64 || dim == 128 || dim == 256) && vdim % 32 == 0 && vdim >= 32 && vdim <= 256 && page_shift >= 6 && ldq % 4 == 0;
 }
 
 void launch_gqa_mfma(tgx_ctx* c, const tgx::StepMeta& m, const tgx::GqaMfmaArgs& a, dim3 grid, bool split) {
