@@ -26,6 +26,8 @@ struct StackGemmArgs {
   int M, N, K;
   float scale;                 // SG_STORE: C = acc * scale + bias
   const float* bias;           // SG_STORE: [N] per z (column z * c_zoff + n), nullptr: none
+  int gate_col0, gate_heads;   // SG_STORE: columns [gate_col0, + gate_heads) leave as log input gates cap tanh(v / cap), the next gate_heads columns as log forget gates
+  float gate_cap;              //           logsigmoid(cap tanh(v / cap)) (the two gate rows of a matrix-memory layer's input product); gate_heads 0: none
   float limit;                 // SG_EXPERT_ACT
   const float* G; long long ldg; int g_col0;     // SG_GATE: C = acc * sigmoid(G[row][g_col0 + z * c_zoff + n])
   const float* rw;             // SG_ROWSCALE: C = acc * rw[c row]
@@ -36,6 +38,14 @@ struct StackGemmArgs {
 __device__ __forceinline__ float expert_act(float gate, float up, float limit) {
   const float g = fminf(gate, limit), u = fminf(fmaxf(up, -limit), limit);
   return g / (1.0f + expf(-1.702f * g)) * (u + 1.0f);
+}
+// log-space gates of a matrix-memory layer: soft cap, and log sigmoid in the form that loses nothing for large |z|
+__device__ __forceinline__ float soft_cap(float z, float cap) { return cap * tanhf(z / cap); }
+__device__ __forceinline__ float log_sigmoid(float z) { return fminf(z, 0.f) - log1pf(expf(-fabsf(z))); }
+__device__ __forceinline__ float store_value(const StackGemmArgs& a, float v, size_t bias_at, int n) {
+  float o = a.bias ? fmaf(v, a.scale, a.bias[bias_at]) : v * a.scale;
+  if (a.gate_heads > 0 && n >= a.gate_col0) { o = soft_cap(o, a.gate_cap); if (n >= a.gate_col0 + a.gate_heads) o = log_sigmoid(o); }
+  return o;
 }
 // the plain gated expert: silu(gate) * up
 __device__ __forceinline__ float silu_mul(float gate, float up) { return gate / (1.0f + expf(-gate)) * up; }
@@ -222,7 +232,7 @@ __global__ __launch_bounds__(256) void stack_gemm_kernel(const StackGemmArgs a) 
         const int n = n0 + wn * (32 * WT) + j * 32 + (lane & 31);
         if (n >= a.N) continue;
         const float v = acc[0][i][j][r];
-        if constexpr (EPI == SG_STORE) cp[n] = a.bias ? fmaf(v, a.scale, a.bias[(size_t)z * a.c_zoff + n]) : v * a.scale;
+        if constexpr (EPI == SG_STORE) cp[n] = store_value(a, v, (size_t)z * a.c_zoff + n, n);
         else if constexpr (EPI == SG_ADD) cp[n] += v;
         else if constexpr (EPI == SG_GATE) cp[n] = v / (1.0f + expf(-a.G[crow * a.ldg + a.g_col0 + (size_t)z * a.c_zoff + n]));
         else if constexpr (EPI == SG_EXPERT_ACT) cp[n] = expert_act(v, acc[NB - 1][i][j][r], a.limit);
@@ -320,7 +330,7 @@ __global__ __launch_bounds__(256) void stack_gemv_kernel(const StackGemmArgs a) 
       const int n = n0 + j;
       if (n >= a.N) break;
       const float v = acc[0][j][r];
-      if constexpr (EPI == SG_STORE) cp[n] = a.bias ? fmaf(v, a.scale, a.bias[(size_t)z * a.c_zoff + n]) : v * a.scale;
+      if constexpr (EPI == SG_STORE) cp[n] = store_value(a, v, (size_t)z * a.c_zoff + n, n);
       else if constexpr (EPI == SG_ADD) cp[n] += v;
       else if constexpr (EPI == SG_GATE) cp[n] = v / (1.0f + expf(-a.G[crow * a.ldg + a.g_col0 + (size_t)z * a.c_zoff + n]));
       else if constexpr (EPI == SG_EXPERT_ACT) cp[n] = expert_act(v, acc[NB - 1][j][r], a.limit);

@@ -13,6 +13,7 @@
 //   router_group_kernel     softmax scores, correction, group limit, top-k, weights = scores * scale; the shared expert's gate
 #pragma once
 #include "stack.h"
+#include "stack_gemm.h"
 
 namespace tgx {
 
@@ -254,15 +255,15 @@ __global__ __launch_bounds__(256) void gqa_attn_merge_kernel(GqaAttnArgs a) {
 // One workgroup per (entry, head, 4 CW value columns; CW = 16, or 8 when the step has few entries and heads) walks the entry's tokens in order, a block of
 // 8 .. 32 at a time:
 //   stage   q (scaled), k, the workgroup's v columns and the gate pre-activations of the block's tokens into LDS (coalesced)
-//   gates   one thread per token: i, f, then mx' and the three factors exp(f + mx - mx'), exp(i - mx'), exp(-mx') from prefix sums over the block
-//           (mx'_t = B_t + max(mx_before, max_{s<=t} (i_s - B_s)), B_t = f_0 + .. + f_t: the recurrence unrolled)
+//   gates   one lane per token: mx' and the three factors exp(f + mx - mx'), exp(i - mx'), exp(-mx') from prefix sums and maxima over the block
+//           (mx'_t = B_t + max(mx_before, max_{s<=t} (i_s - B_s)), B_t = f_0 + .. + f_t: the recurrence unrolled); i and f arrive activated
 //   scan    no barrier and no lane exchange inside: a wave owns CW columns, its lanes = 64 / CW row groups x CW columns, each lane keeps DPER rows of its
 //           column in registers and leaves its partial sums of S^T q and n . q (every wave computes the latter) per token in LDS
 //   out     the partial sums of the block's tokens are added up (over the row groups; over the wave for n . q) and divided
 // n and mx are double-buffered per slot (buffer `par` is read, `par ^ 1` written), because the workgroups of a head's other columns read them too.
 // The outputs leave un-normed (mlstm_out_kernel follows).
 struct MlstmArgs {
-  const float* proj; long long ldp;     // [T][q | k | v | g | zi | zf]: q, k per head [dim]; v, g per head [vdim]; zi, zf per head (biases added)
+  const float* proj; long long ldp;     // [T][q | k | v | g | i | f]: q, k per head [dim]; v, g per head [vdim]; i, f per head: the log gates (the input product's epilogue has applied cap and log sigmoid)
   int heads, dim, vdim;
   float cap, qscale;
   float* S;                             // [slots][heads][dim][vdim]
@@ -271,7 +272,6 @@ struct MlstmArgs {
   size_t n_buf, mx_buf;                 // elements between the two buffers
   float* hs; long long ldh;             // [T][heads * vdim]
 };
-__device__ __forceinline__ float log_sigmoid(float z) { return fminf(z, 0.f) - log1pf(expf(-fabsf(z))); }
 template <int DPER, int CW>      // rows per lane and columns per wave: (64 / CW) DPER >= dim
 __global__ __launch_bounds__(256) void mlstm_scan_kernel(StepMeta m, MlstmArgs a) {
   constexpr int RG = 64 / CW, NPL = (DPER + CW - 1) / CW, DP = RG * DPER, LP = DPER + 4, CB = 4 * CW;      // LP: a row group's LDS stride (the groups' reads fall into different banks)
@@ -327,20 +327,23 @@ __global__ __launch_bounds__(256) void mlstm_scan_kernel(StepMeta m, MlstmArgs a
     }
 #pragma unroll
     for (int u = 0; u < NV; u++) { const int i = tid + 256 * u; if (i < TB * CB) s_v[i / CB][i % CB] = rv[u]; }
-    if (tid < nb) { s_zi[tid] = a.cap * tanhf(rzi / a.cap); s_zf[tid] = log_sigmoid(a.cap * tanhf(rzf / a.cap)); }
+    if (tid < TB) { s_zi[tid] = tid < nb ? rzi : -INFINITY; s_zf[tid] = tid < nb ? rzf : 0.f; }
     __syncthreads();
     if (t0 + TB < cnt) fetch(t0 + TB);
-    if (tid < nb) {
-      const float mprev = s_mx[blk & 1];
-      float bs = 0.f, c = -INFINITY, mbefore = mprev;      // mbefore: the maximum after token tid - 1
-      for (int s2 = 0; s2 <= tid; s2++) {
-        if (s2 == tid) mbefore = s2 == 0 ? mprev : bs + fmaxf(mprev, c);
-        bs += s_zf[s2];
-        c = fmaxf(c, s_zi[s2] - bs);
-      }
+    if (wv == 0) {      // one lane per token: prefix sums of the log forget gates, prefix maxima of i - B, both by lane exchanges
+      const float fl = lane < TB ? s_zf[lane] : 0.f, ig = lane < TB ? s_zi[lane] : -INFINITY, mprev = s_mx[blk & 1];
+      float bs = fl;
+#pragma unroll
+      for (int o = 1; o < TB; o <<= 1) { const float v = __shfl_up(bs, o, 64); if (lane >= o) bs += v; }
+      float c = ig - bs;
+#pragma unroll
+      for (int o = 1; o < TB; o <<= 1) { const float v = __shfl_up(c, o, 64); if (lane >= o) c = fmaxf(c, v); }
       const float mn = bs + fmaxf(mprev, c);
-      s_keep[tid] = expf(s_zf[tid] + mbefore - mn); s_take[tid] = expf(s_zi[tid] - mn); s_emn[tid] = expf(-mn);
-      if (tid == nb - 1) s_mx[(blk + 1) & 1] = mn;
+      const float up = __shfl_up(mn, 1, 64), mbefore = lane == 0 ? mprev : up;      // the maximum after the token before
+      if (lane < nb) {
+        s_keep[lane] = expf(fl + mbefore - mn); s_take[lane] = expf(ig - mn); s_emn[lane] = expf(-mn);
+        if (lane == nb - 1) s_mx[(blk + 1) & 1] = mn;
+      }
     }
     __syncthreads();
     for (int t = 0; t < nb; t++) {

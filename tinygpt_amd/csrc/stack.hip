@@ -402,9 +402,10 @@ int run_mlstm(tgx_ctx* c, const tgx::StepMeta& m, StackLayerW& w, const float* h
   StackModel* sm = c->stack;
   const tgx_layer_desc& ld = w.d;
   const int W = sm->d.width, H = ld.heads, qd = H * ld.dim, vd = H * ld.vdim, nin = 2 * qd + 2 * vd + 2 * H;
-  // [q | k | v | gate | zi | zf] = h . w_in^T (+ the gate biases)
+  // [q | k | v | gate | i | f] = h . w_in^T (+ the gate biases); i and f through the soft cap (and the log sigmoid) in the product's epilogue
   tgx::StackGemmArgs g{};
   g.A = hin; g.lda = W; g.B = w.w_in; g.ldb = W; g.C = sm->proj; g.ldc = nin; g.M = T; g.N = nin; g.K = W; g.scale = 1.f; g.bias = w.b_in;
+  g.gate_col0 = 2 * qd + 2 * vd; g.gate_heads = H; g.gate_cap = ld.gate_cap;      // the two gate rows leave the product as log gates
   launch_gemm(c, g, tgx::SG_STORE, 1);
   tgx::MlstmArgs ma{};
   ma.proj = sm->proj; ma.ldp = nin; ma.heads = H; ma.dim = ld.dim; ma.vdim = ld.vdim; ma.cap = ld.gate_cap; ma.qscale = 1.0f / sqrtf((float)ld.dim);
