@@ -9,7 +9,8 @@
 //      starts at exp(sink) where the design has a sink: a term without key or value), P as two 16-bit terms and the rows' rescale factors back to LDS
 //   3. O += P V: every wave owns 32 NT of the vdim output columns; its B operand comes from a TRANSPOSED copy of the value page ([channel][token]: eight
 //      consecutive keys of a channel are one 16-byte load) that the append kernel writes
-// Q (score scale folded in) enters as two 16-bit terms (one with option act.round16).  Key tiles never straddle a page (pages hold a multiple of 64
+// Q (score scale and log2 e folded in: the softmax runs in base 2 on the hardware exponential, as in the other families' prompt attention) enters as two 16-bit
+// terms (one with option act.round16).  Key tiles never straddle a page (pages hold a multiple of 64
 // tokens).  The output is multiplied by sigmoid(gate) where a gate is given.  SPLIT: blockIdx.z takes a range of the keys and leaves (m, l, O) records
 // for gqa_attn_merge_kernel.
 #pragma once
@@ -32,6 +33,8 @@ struct GqaMfmaArgs {
 template <int DT, int ND, int NT, bool SPLIT>      // ND = dim / 64: 16-channel steps of a wave's share of the contraction; NT = ceil(vdim / 128): 32-column output tiles per wave
 __global__ __launch_bounds__(256) void gqa_attn_mfma_kernel(StepMeta m, GqaMfmaArgs a) {
   constexpr int RQ = 16 * ND, KS = ND;
+  constexpr float LOG2E = 1.4426950408889634f, LN2 = 0.6931471805599453f;
+  const float qscale = a.scale * LOG2E;
   __shared__ float s_part[4][32][65];
   __shared__ __attribute__((aligned(16))) bf16_t s_ph[32][72], s_pl[32][72];
   __shared__ float s_corr[32], s_l[32];
@@ -58,7 +61,7 @@ __global__ __launch_bounds__(256) void gqa_attn_mfma_kernel(StepMeta m, GqaMfmaA
       const f32x4 v0 = *reinterpret_cast<const f32x4*>(qp + 16 * kk), v1 = *reinterpret_cast<const f32x4*>(qp + 16 * kk + 4);
       bf16_t h[8], l[8];
 #pragma unroll
-      for (int i = 0; i < 4; i++) { split16<DT>(r < nrows ? v0[i] * a.scale : 0.f, h[i], l[i]); split16<DT>(r < nrows ? v1[i] * a.scale : 0.f, h[4 + i], l[4 + i]); }
+      for (int i = 0; i < 4; i++) { split16<DT>(r < nrows ? v0[i] * qscale : 0.f, h[i], l[i]); split16<DT>(r < nrows ? v1[i] * qscale : 0.f, h[4 + i], l[4 + i]); }
       u32x4 uh, ul;
 #pragma unroll
       for (int i = 0; i < 4; i++) { uh[i] = (unsigned int)h[2 * i] | ((unsigned int)h[2 * i + 1] << 16); ul[i] = (unsigned int)l[2 * i] | ((unsigned int)l[2 * i + 1] << 16); }
@@ -77,7 +80,7 @@ __global__ __launch_bounds__(256) void gqa_attn_mfma_kernel(StepMeta m, GqaMfmaA
   const bool svalid = sr < nrows;
   const int skeys = svalid ? past + sr / Gq + 1 : 0;
   const bool sinked = a.has_sink && svalid && (!SPLIT || blockIdx.z == 0);
-  float m_s = sinked ? a.sink : -INFINITY, l_s = sinked ? 1.f : 0.f;
+  float m_s = sinked ? a.sink * LOG2E : -INFINITY, l_s = sinked ? 1.f : 0.f;      // the running maximum in base-2 units
 
   auto key_rows = [&](int kt) -> const bf16_t* {
     const size_t pg = (size_t)m.tbl[(size_t)slot * m.tbl_stride + (kt >> m.page_shift)];
@@ -135,11 +138,11 @@ __global__ __launch_bounds__(256) void gqa_attn_mfma_kernel(StepMeta m, GqaMfmaA
       tmax = fmaxf(tmax, __shfl_xor(tmax, 1, 64)); tmax = fmaxf(tmax, __shfl_xor(tmax, 2, 64)); tmax = fmaxf(tmax, __shfl_xor(tmax, 4, 64));
       const float mn = fmaxf(m_s, tmax);
       const bool dead = mn == -INFINITY;                  // nothing seen yet (a row of another split, or a padding row)
-      const float corr = dead ? 1.f : expf(m_s - mn);
+      const float corr = dead ? 1.f : __builtin_amdgcn_exp2f(m_s - mn);
       float psum = 0.f;
       bf16_t ph[8], pl[8];
 #pragma unroll
-      for (int c = 0; c < 8; c++) { const float p = dead ? 0.f : expf(sv[c] - mn); psum += p; split16<DT>(p, ph[c], pl[c]); }
+      for (int c = 0; c < 8; c++) { const float p = dead ? 0.f : __builtin_amdgcn_exp2f(sv[c] - mn); psum += p; split16<DT>(p, ph[c], pl[c]); }
       psum += __shfl_xor(psum, 1, 64); psum += __shfl_xor(psum, 2, 64); psum += __shfl_xor(psum, 4, 64);
       l_s = fmaf(l_s, corr, psum);
       m_s = mn;
@@ -179,7 +182,7 @@ __global__ __launch_bounds__(256) void gqa_attn_mfma_kernel(StepMeta m, GqaMfmaA
   };
   if ((lane & 7) == 0) {
     s_l[srow] = l_s;
-    if (SPLIT && svalid) { float* rec = rec_of(sr); rec[0] = m_s; rec[1] = l_s; }
+    if (SPLIT && svalid) { float* rec = rec_of(sr); rec[0] = m_s * LN2; rec[1] = l_s; }      // the merge kernel works in natural units
   }
   __syncthreads();
 #pragma unroll
