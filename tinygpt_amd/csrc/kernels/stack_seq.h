@@ -250,7 +250,7 @@ __global__ __launch_bounds__(256) void gqa_attn_merge_kernel(GqaAttnArgs a) {
 }
 
 // ---- matrix memory (mLSTM).  Per head: a [dim][vdim] matrix S, a [dim] vector n and a running maximum mx (log scale), all fp32, all zero (mx too) at a
-// sequence's start.  For every token, with log gates i = cap tanh(zi / cap), f = logsigmoid(cap tanh(zf / cap)):
+// sequence's start.  For every token, with log gates i = cap tanh(zi / cap), f = logsigmoid(cap tanh(zf / cap)) (applied by the input product's epilogue):
 //   mx' = max(f + mx, i);  S' = exp(f + mx - mx') S + exp(i - mx') k v^T;  n' likewise with k;  o = S'^T q / (max(|n' . q|, exp(-mx')) + 1e-6)
 // One workgroup per (entry, head, 4 CW value columns; CW = 16, or 8 when the step has few entries and heads) walks the entry's tokens in order, a block of
 // 8 .. 32 at a time:
@@ -265,7 +265,7 @@ __global__ __launch_bounds__(256) void gqa_attn_merge_kernel(GqaAttnArgs a) {
 struct MlstmArgs {
   const float* proj; long long ldp;     // [T][q | k | v | g | i | f]: q, k per head [dim]; v, g per head [vdim]; i, f per head: the log gates (the input product's epilogue has applied cap and log sigmoid)
   int heads, dim, vdim;
-  float cap, qscale;
+  float qscale;
   float* S;                             // [slots][heads][dim][vdim]
   float* n;                             // [2][slots][heads][dim]
   float* mx;                            // [2][slots][heads]

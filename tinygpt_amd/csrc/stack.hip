@@ -408,7 +408,7 @@ int run_mlstm(tgx_ctx* c, const tgx::StepMeta& m, StackLayerW& w, const float* h
   g.gate_col0 = 2 * qd + 2 * vd; g.gate_heads = H; g.gate_cap = ld.gate_cap;      // the two gate rows leave the product as log gates
   launch_gemm(c, g, tgx::SG_STORE, 1);
   tgx::MlstmArgs ma{};
-  ma.proj = sm->proj; ma.ldp = nin; ma.heads = H; ma.dim = ld.dim; ma.vdim = ld.vdim; ma.cap = ld.gate_cap; ma.qscale = 1.0f / sqrtf((float)ld.dim);
+  ma.proj = sm->proj; ma.ldp = nin; ma.heads = H; ma.dim = ld.dim; ma.vdim = ld.vdim; ma.qscale = 1.0f / sqrtf((float)ld.dim);
   ma.S = w.mS; ma.n = w.mn; ma.mx = w.mm; ma.n_buf = (size_t)sm->d.max_seqs * H * ld.dim; ma.mx_buf = (size_t)sm->d.max_seqs * H;
   ma.hs = sm->hs; ma.ldh = vd;
   // columns per wave: 16, or 8 (twice the workgroups, half the rows per lane) while the step's entries and heads leave most of the chip idle
